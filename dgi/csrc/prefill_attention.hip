@@ -106,7 +106,7 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void prefill_attn_kernel(
     // merges "Q pending" from the preheader into the loop header and, to reach the older Q
     // loads, emits vmcnt(0) before the first QK^T MFMA of EVERY tile — which also waits for
     // the K/V loads of tile i+2 issued a few instructions earlier: one full HBM round trip
-    // per tile and no load/compute overlap at all (round 5 disassembly).
+    // per tile and no load/compute overlap at all.
     __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0), expcnt / lgkmcnt untouched (gfx9 encoding)
   }
 
