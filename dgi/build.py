@@ -47,32 +47,46 @@ def _run(cmd):
     return r
 
 
-def build(verbose: bool = False, force: bool = False) -> str:
-    os.makedirs(BUILD, exist_ok=True)
+# hipcc device-code flags: no packed-fp32 VALU forms (the compiler otherwise makes them from
+# ordinary float code); the host pass warns that it does not know the feature, harmlessly
+DEVICE_FLAGS = ["-munsafe-fp-atomics", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+
+# extension libraries: name -> (source folder, output).  "core" is every kernel of the Llama-family
+# runtime (dgi/_C.so); "mix" the mixer-block kernels of the per-layer-geometry models
+# (dgi/_C_mix.so: norms, q/k norm + rotary, masked attention, activations), which builds in
+# seconds so a model that needs only those does not wait for the big GEMM kernels.
+GROUPS = {"core": (CSRC, OUT), "mix": (os.path.join(CSRC, "mix"), os.path.join(HERE, "_C_mix.so"))}
+
+
+def build(verbose: bool = False, force: bool = False, group: str = "core") -> str:
+    src_dir, out = GROUPS[group]
+    obj_dir = BUILD if group == "core" else BUILD + "_" + group
+    os.makedirs(obj_dir, exist_ok=True)
     inc, lib, abi = _torch_paths()
     hdrs = [os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith(".h")]
-    kernels = sorted(f for f in os.listdir(CSRC) if f.endswith(".hip"))
+    hdrs += [os.path.join(src_dir, f) for f in os.listdir(src_dir) if f.endswith(".h") and src_dir != CSRC]
+    kernels = sorted(f for f in os.listdir(src_dir) if f.endswith(".hip"))
     common = ["-O3", "-fPIC", "-std=c++17", f"-D_GLIBCXX_USE_CXX11_ABI={abi}"]
     jobs = []
     objs = []
     for k in kernels:
-        src = os.path.join(CSRC, k)
-        obj = os.path.join(BUILD, k + ".o")
+        src = os.path.join(src_dir, k)
+        obj = os.path.join(obj_dir, k + ".o")
         objs.append(obj)
         if force or _newer([src] + hdrs, obj):
-            jobs.append([HIPCC, f"--offload-arch={ARCH}", *common, "-munsafe-fp-atomics", "-c", src, "-o", obj])
-    bsrc = os.path.join(CSRC, "bindings.cpp")
-    bobj = os.path.join(BUILD, "bindings.o")
+            jobs.append([HIPCC, f"--offload-arch={ARCH}", *common, *DEVICE_FLAGS, "-c", src, "-o", obj])
+    bsrc = os.path.join(src_dir, "bindings.cpp")
+    bobj = os.path.join(obj_dir, "bindings.o")
     objs.append(bobj)
     py_inc = sysconfig.get_paths()["include"]
     if force or _newer([bsrc], bobj):
         jobs.append([HIPCC, *common, "-D__HIP_PLATFORM_AMD__=1", "-DUSE_ROCM=1", "-DTORCH_EXTENSION_NAME=_C",
                      *[f"-I{p}" for p in inc], f"-I{py_inc}", "-I/opt/rocm/include", "-x", "c++", "-c", bsrc, "-o", bobj])
     # native runtime pieces (C++ only)
-    for f in sorted(os.listdir(CSRC)):
+    for f in sorted(os.listdir(src_dir)):
         if f.endswith(".cc"):
-            src = os.path.join(CSRC, f)
-            obj = os.path.join(BUILD, f + ".o")
+            src = os.path.join(src_dir, f)
+            obj = os.path.join(obj_dir, f + ".o")
             objs.append(obj)
             if force or _newer([src] + hdrs, obj):
                 jobs.append(["g++", *common, f"-I{py_inc}", *[f"-I{p}" for p in inc], "-c", src, "-o", obj])
@@ -81,10 +95,12 @@ def build(verbose: bool = False, force: bool = False) -> str:
         for r in ex.map(_run, jobs):
             if verbose and r.stderr:
                 print(r.stderr, file=sys.stderr)
-    if force or jobs or not os.path.exists(OUT):
-        _run([HIPCC, "-shared", "-fPIC", f"--offload-arch={ARCH}", *objs, "-o", OUT, f"-L{lib}",
+    if force or jobs or not os.path.exists(out):
+        tmp = out + f".tmp{os.getpid()}"
+        _run([HIPCC, "-shared", "-fPIC", f"--offload-arch={ARCH}", *objs, "-o", tmp, f"-L{lib}",
               "-lc10", "-lc10_hip", "-ltorch", "-ltorch_cpu", "-ltorch_hip", f"-Wl,-rpath,{lib}"])
-    return OUT
+        os.replace(tmp, out)
+    return out
 
 
 SHM_SRC = os.path.join(CSRC, "host", "shm_ring.cc")
@@ -134,5 +150,6 @@ if __name__ == "__main__":
             print(build_sanitized(k, force="--force" in sys.argv))
         sys.exit(0)
     print(build_shm(force="--force" in sys.argv))
-    p = build(verbose=True, force="--force" in sys.argv)
-    print(p)
+    groups = [g for g in GROUPS if g in sys.argv] or list(GROUPS)
+    for g in groups:
+        print(build(verbose=True, force="--force" in sys.argv, group=g))

@@ -17,7 +17,7 @@ import torch
 
 from dgi.kv.block_pool import BlockPool, OutOfBlocks, num_blocks_for_budget
 from dgi.models.config import ModelConfig, get_config
-from dgi.models.llama import LlamaModel
+from dgi.models import build_model
 from dgi.runtime.model_runner import ModelRunner
 from dgi.sched.request import Request, SamplingParams, Status
 from dgi.sched.scheduler import Scheduler, SchedulerConfig
@@ -78,7 +78,12 @@ def engine_block_budget(cfg: EngineConfig, mc: ModelConfig, n_local: int, device
         budget = max(0, _device_free_bytes(device) - cfg.workspace_bytes) * cfg.kv_fraction
     else:
         budget = 1 << 30  # CPU rehearsal runs: a fixed 1 GiB pool
-    nblocks = num_blocks_for_budget(int(budget), max(1, n_local), mc.num_kv_heads, mc.head_dim, cfg.block_size)
+    es = torch.tensor([], dtype=cfg.dtype).element_size()
+    if hasattr(mc, "kv_layer_shapes"):
+        per_block = max(1, mc.kv_bytes_per_token(es, layers=None) * cfg.block_size)
+        nblocks = int(budget // per_block)
+    else:
+        nblocks = num_blocks_for_budget(int(budget), max(1, n_local), mc.num_kv_heads, mc.head_dim, cfg.block_size, es)
     # never more than what max_num_seqs full-length sequences can use (+ prefix cache room)
     cap = 2 * cfg.max_num_seqs * ((cfg.max_model_len + cfg.block_size - 1) // cfg.block_size) + 1
     return max(2, min(nblocks, cap))
@@ -115,16 +120,19 @@ class LLMEngine:
         self.model_cfg = model_cfg or get_config(self.checkpoint or cfg.model)
         self.model_cfg.max_position = max(self.model_cfg.max_position, cfg.max_model_len)
         t0 = time.perf_counter()
-        self.model = model or LlamaModel(self.model_cfg, self.device, cfg.dtype, cfg.layer_start, cfg.layer_end,
-                                         seed=cfg.seed, checkpoint=self.checkpoint)
+        self.model = model or build_model(self.model_cfg, self.device, cfg.dtype, cfg.layer_start, cfg.layer_end,
+                                          seed=cfg.seed, checkpoint=self.checkpoint)
         if self.device.type == "cuda":
             torch.cuda.synchronize()
         self.load_seconds = time.perf_counter() - t0
         mc = self.model_cfg
         n_local = self.model.num_local_layers
         nblocks = engine_block_budget(cfg, mc, n_local, self.device)
+        shapes = None
+        if hasattr(mc, "kv_layer_shapes"):          # per-layer page geometry (dgi.kv.block_pool)
+            shapes = mc.kv_layer_shapes(self.model.layer_start, self.model.layer_end) or None
         self.pool = BlockPool(nblocks, cfg.block_size, max(1, n_local), mc.num_kv_heads, mc.head_dim,
-                              cfg.dtype, self.device)
+                              cfg.dtype, self.device, layer_shapes=shapes)
         align = cfg.token_align if cfg.token_align >= 0 else (256 if self.device.type == "cuda" else 0)
         self.scheduler = Scheduler(self.pool, SchedulerConfig(cfg.max_num_seqs, cfg.max_num_batched_tokens,
                                                               cfg.max_model_len, cfg.enable_prefix_caching,
@@ -172,7 +180,8 @@ class LLMEngine:
                       "finished": 0, "step_time": 0.0}
         # MLP row padding measured on this GPU (hipBLASLt kernel-selection cliffs, dgi.runtime.gemm_pad)
         self.mlp_pad_table = None
-        if self.device.type == "cuda" and getattr(self.model, "mlp_pad", None) is None:
+        if self.device.type == "cuda" and getattr(self.model, "mlp_pad", None) is None \
+                and getattr(self.model, "routes_gemms", True):
             from dgi.runtime.gemm_pad import build_for_model
             t1 = time.perf_counter()
             self.mlp_pad_table = build_for_model(self.model, cfg.max_num_batched_tokens)
@@ -251,7 +260,10 @@ class LLMEngine:
             outs = self._step_mixed_lookahead()
             self._account(n, time.perf_counter() - t0)
             return outs
-        self.model.kv_cache = self.pool.kv   # engines may share one model object
+        if hasattr(self.model, "attach_cache"):   # engines may share one model object
+            self.model.attach_cache(self.pool)
+        else:
+            self.model.kv_cache = self.pool.kv
         with phase("schedule"):
             sbud = self.step_budget
             cap = None
@@ -445,6 +457,78 @@ class LLMEngine:
             # (its tokens are discarded) instead of leaving the engine with work and no requests
             self.drain()
         return outs
+
+    # ------------------------------------------------------------------ teacher-forced replay
+    def feed(self, entries, end=()) -> list:
+        """One step over GIVEN tokens: ``entries`` is [(rid, tokens, want)], each request's next
+        tokens and the offsets among them whose logits are asked for; returns one fp32 host
+        tensor [len(want), vocab] per entry.  Nothing is sampled.  All entries run as one batch
+        through the scheduler, the block pool and the model's step: a request is admitted at
+        its first entry, a single token of a request that already holds tokens is a decode row,
+        anything else a prompt portion; requests not named in a step keep their pages and sit
+        it out.  ``end``: request ids released after the step (their pages return to the pool).
+        Needs an engine without prefix caching (a cached prefix is not recomputed, so its
+        logits could not be returned)."""
+        sch = self.scheduler
+        if sch.radix is not None:
+            raise RuntimeError("feed() needs enable_prefix_caching=False")
+        if self._la is not None or self._mx is not None:
+            self.drain()
+        named = {}
+        for rid, toks, want in entries:
+            toks = [int(t) for t in toks]
+            if not toks or rid in named:
+                raise ValueError("feed(): every entry brings tokens, one entry per request and step")
+            req = self.requests.get(rid)
+            if req is None:
+                req = Request(toks, SamplingParams(max_tokens=1 << 30, temperature=0.0, ignore_eos=True), rid=rid)
+                sch.add(req)
+                self.requests[rid] = req
+            else:
+                if req.total_len + len(toks) >= self.cfg.max_model_len:
+                    raise ValueError(f"request {rid!r} exceeds max_model_len {self.cfg.max_model_len}")
+                req.prompt.extend(toks)
+            # one token on top of cached ones: a decode row (prefill_target == num_computed)
+            req.prefill_target = req.num_computed if (len(toks) == 1 and req.num_computed > 0) else len(req.prompt)
+            named[rid] = (req, len(toks), sorted(int(w) for w in want))
+        for r in sch.running:
+            r.busy = r.rid not in named
+        try:
+            if hasattr(self.model, "attach_cache"):
+                self.model.attach_cache(self.pool)
+            sb = sch.schedule(preempt=False)
+        finally:
+            for r in sch.running:
+                r.busy = False
+        dec_row = {r.rid: i for i, r in enumerate(sb.decode)}
+        chunk = {c.req.rid: c for c in sb.prefill}
+        for rid, (req, n, want) in named.items():
+            c = chunk.get(rid)
+            if not ((rid in dec_row and n == 1) or (c is not None and c.length == n)):
+                raise RuntimeError(f"feed(): request {rid!r} did not fit this step (pool pages or token budget)")
+            if c is not None:
+                c.logit_pos = want
+        logits = self.runner.execute_logits(sb)
+        self._advance(sb)
+        out = []
+        row = len(sb.decode)
+        first = {}
+        for c in sb.prefill:
+            first[c.req.rid] = row
+            row += len(c.logit_pos or ())
+        for rid, _toks, _want in entries:
+            req, n, want = named[rid]
+            if rid in dec_row:
+                out.append(logits[dec_row[rid]: dec_row[rid] + 1] if want else logits[:0])
+            else:
+                out.append(logits[first[rid]: first[rid] + len(want)])
+            req.prefill_target = req.num_computed
+        for rid in end:
+            req = self.requests.pop(rid, None)
+            if req is not None:
+                sch.finish(req, "stop")
+                self.stats["finished"] += 1
+        return out
 
     def _apply(self, sb, rows, tokens) -> list[StepOutput]:
         """Commit one executed batch: advance KV cursors, append tokens, stop checks."""

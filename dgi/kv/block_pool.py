@@ -11,6 +11,14 @@ kv_cache.py:130-139, which its own tests contradict).
 Sizing for MI355X: ``num_blocks_for_budget`` turns a byte budget (288 GB HBM
 minus weights and activation workspace, times ``kv_fraction``) into a block
 count.
+
+Models whose layers differ in cache geometry (kv heads, key size, value size per layer)
+pass ``layer_shapes``: the pool then owns one flat allocation cut into per-layer
+``k [num_blocks, n_kv, bs, dk]`` and ``v [num_blocks, n_kv, bs, dv]`` views (``layers``).  A
+block id still names the page of every layer, so allocation, reference counts, the
+scheduler and the radix cache are the same; ``kv`` (the single 6-D tensor that the
+host tier and cross-worker transfer move) exists only when all layers share one geometry
+with dk == dv.
 """
 from __future__ import annotations
 
@@ -31,18 +39,46 @@ def num_blocks_for_budget(budget_bytes: int, num_layers: int, num_kv_heads: int,
 
 class BlockPool:
     def __init__(self, num_blocks: int, block_size: int = 16, num_layers: int = 1, num_kv_heads: int = 1,
-                 head_dim: int = 128, dtype=torch.bfloat16, device="cpu", allocate: bool = True):
+                 head_dim: int = 128, dtype=torch.bfloat16, device="cpu", allocate: bool = True,
+                 layer_shapes: Optional[list] = None):
         self.num_blocks = num_blocks
         self.block_size = block_size
+        if layer_shapes is not None:
+            layer_shapes = [tuple(int(x) for x in sh) for sh in layer_shapes]
+            num_layers = len(layer_shapes)
+            if len(set(layer_shapes)) == 1 and layer_shapes[0][1] == layer_shapes[0][2]:
+                num_kv_heads, head_dim = layer_shapes[0][0], layer_shapes[0][1]     # one geometry: the 6-D tensor
+                self.layer_shapes = None
+            else:
+                self.layer_shapes = layer_shapes
+                num_kv_heads = max(g for g, _dk, _dv in layer_shapes)
+                head_dim = max(max(dk, dv) for _g, dk, dv in layer_shapes)
+        else:
+            self.layer_shapes = None
         self.num_layers = num_layers
         self.num_kv_heads = num_kv_heads
         self.head_dim = head_dim
         self.dtype = dtype
         self.device = torch.device(device)
         self.kv: Optional[torch.Tensor] = None
-        if allocate:
+        self.layers: list = []          # per layer (k [NB, n_kv, bs, dk], v [NB, n_kv, bs, dv])
+        self._store: Optional[torch.Tensor] = None
+        if allocate and self.layer_shapes is None:
             self.kv = torch.zeros(num_layers, 2, num_blocks, num_kv_heads, block_size, head_dim,
                                   dtype=dtype, device=self.device)
+            self.layers = [(self.kv[l, 0], self.kv[l, 1]) for l in range(num_layers)]
+        elif allocate:
+            # every region starts on a 256-byte boundary (16-byte vector loads of any row)
+            al = 128
+            offs, n = [], 0
+            for g, dk, dv in self.layer_shapes:
+                for d in (dk, dv):
+                    offs.append((n, g, d))
+                    n += (num_blocks * g * block_size * d + al - 1) // al * al
+            self._store = torch.zeros(n, dtype=dtype, device=self.device)
+            views = [self._store[o: o + num_blocks * g * block_size * d].view(num_blocks, g, block_size, d)
+                     for o, g, d in offs]
+            self.layers = [(views[2 * l], views[2 * l + 1]) for l in range(num_layers)]
         # block 0 is reserved as a scratch/padding page (graph padding rows write there)
         self._free: list[int] = list(range(num_blocks - 1, 0, -1))
         self.ref = [0] * num_blocks
@@ -60,8 +96,10 @@ class BlockPool:
         return self.num_blocks - 1 - len(self._free)
 
     def page_bytes(self) -> int:
-        return 2 * self.num_layers * self.num_kv_heads * self.block_size * self.head_dim * \
-            torch.tensor([], dtype=self.dtype).element_size()
+        es = torch.tensor([], dtype=self.dtype).element_size()
+        if self.layer_shapes is not None:
+            return sum(g * (dk + dv) for g, dk, dv in self.layer_shapes) * self.block_size * es
+        return 2 * self.num_layers * self.num_kv_heads * self.block_size * self.head_dim * es
 
     def can_allocate(self, n: int) -> bool:
         return n <= len(self._free) or (self.evictor is not None and n <= len(self._free) + self.evictor(0))
@@ -102,6 +140,10 @@ class BlockPool:
             dev = self.kv.device
             ops.kv_copy(self.kv, torch.tensor([block], dtype=torch.int32, device=dev),
                         torch.tensor([nb], dtype=torch.int32, device=dev))
+        else:
+            for k, v in self.layers:
+                k[nb].copy_(k[block])
+                v[nb].copy_(v[block])
         self.free([block])
         self.stats["cow"] += 1
         return nb

@@ -1,1 +1,14 @@
-from dgi.models.config import ModelConfig, PRESETS, get_config  # noqa: F401
+from dgi.models.config import BebovikConfig, ModelConfig, PRESETS, get_config  # noqa: F401
+
+
+def model_class(cfg):
+    """The native model class that serves a configuration (the engine's model registry)."""
+    if isinstance(cfg, BebovikConfig):
+        from dgi.models.bebovik import BebovikModel
+        return BebovikModel
+    from dgi.models.llama import LlamaModel
+    return LlamaModel
+
+
+def build_model(cfg, device, dtype, layer_start: int = 0, layer_end=None, **kw):
+    return model_class(cfg)(cfg, device, dtype, layer_start, layer_end, **kw)

@@ -107,11 +107,179 @@ class ModelConfig:
                            bos_token_id=d.get("bos_token_id", 1), eos_token_id=eos)
 
     @staticmethod
-    def from_file(path: str) -> "ModelConfig":
+    def from_file(path: str):
+        """The configuration a ``config.json`` describes: the class is chosen by the file
+        (``architecture`` names a native design, else the HF ``model_type`` families)."""
         if os.path.isdir(path):
             path = os.path.join(path, "config.json")
         with open(path) as f:
-            return ModelConfig.from_hf_dict(json.load(f), name=os.path.basename(os.path.dirname(path)))
+            d = json.load(f)
+        name = os.path.basename(os.path.dirname(os.path.abspath(path)))
+        arch = d.get("architecture")
+        if isinstance(arch, str) and arch.lower() in NATIVE_CONFIGS:
+            return NATIVE_CONFIGS[arch.lower()](d, name)
+        return ModelConfig.from_hf_dict(d, name=name)
+
+
+@dataclasses.dataclass
+class RotarySpec:
+    """Rotary position parameters of one attention mixer: the first ``dims`` dimensions of a
+    head rotate in interleaved pairs (2i, 2i+1) at frequency base^(-2i/dims); ``scaling``
+    (factor, low, high, original) rescales the frequencies by wavelength, or None."""
+    base: float
+    dims: int
+    scaling: Optional[dict] = None
+
+
+@dataclasses.dataclass
+class AttentionSpec:
+    """One softmax-attention mixer: H query heads over G key/value heads, query/key size
+    ``dim`` and value size ``vdim``; ``mask_kind`` "chunk" limits a query to the keys of its
+    own block of ``mask_size`` positions (counted from position 0), "causal" to all earlier."""
+    heads: int
+    kv_heads: int
+    dim: int
+    vdim: int
+    scale: float
+    rot: Optional[RotarySpec] = None
+    mask_kind: str = "causal"
+    mask_size: int = 0
+    qk_norm: bool = True
+    out_gate: bool = True
+
+    @property
+    def q_size(self) -> int:
+        return self.heads * self.dim
+
+    @property
+    def k_size(self) -> int:
+        return self.kv_heads * self.dim
+
+    @property
+    def v_size(self) -> int:
+        return self.kv_heads * self.vdim
+
+    @property
+    def o_size(self) -> int:
+        return self.heads * self.vdim
+
+
+@dataclasses.dataclass
+class GluSpec:
+    """Dense gated feed-forward: ``ff`` inner width, ``limit`` the clamp of gate and up."""
+    ff: int
+    limit: float
+    kind: str = "dense"
+
+
+@dataclasses.dataclass
+class LayerSpec:
+    type: str
+    mixer: AttentionSpec
+    mlp: Optional[GluSpec] = None
+
+
+@dataclasses.dataclass
+class BebovikConfig:
+    """A Bebovik decoder: per-layer mixer geometry (every size may differ between layers),
+    Dynamic-Tanh norms around both sublayers with layer scale, a scaled embedding with its own
+    norm, and scaled + soft-capped logits.  Built from the design's ``config.json``
+    (``from_dict``) or in code (tests, benchmarks)."""
+    name: str
+    vocab_size: int
+    hidden_size: int
+    layers: list
+    embedding_scale: float = 1.0
+    logit_scale: float = 1.0
+    logit_softcap: float = 0.0
+    norm_eps: float = 1e-6
+    max_position: int = 8192
+    bos_token_id: int = -1
+    eos_token_id: int = -1
+    arch: str = "bebovik"
+    tie_embeddings: bool = False
+
+    # the engine-facing view shared with ModelConfig
+    @property
+    def num_layers(self) -> int:
+        return len(self.layers)
+
+    @property
+    def num_heads(self) -> int:
+        return max(l.mixer.heads for l in self.layers)
+
+    @property
+    def num_kv_heads(self) -> int:
+        return max(l.mixer.kv_heads for l in self.layers)
+
+    @property
+    def head_dim(self) -> int:
+        return max(max(l.mixer.dim, l.mixer.vdim) for l in self.layers)
+
+    @property
+    def rms_eps(self) -> float:
+        return self.norm_eps
+
+    def kv_layer_shapes(self, start: int = 0, end: Optional[int] = None) -> list:
+        """(kv heads, key size, value size) of each layer's cache pages."""
+        return [(l.mixer.kv_heads, l.mixer.dim, l.mixer.vdim) for l in self.layers[start:end]]
+
+    def kv_bytes_per_token(self, dtype_bytes: int = 2, layers: Optional[int] = None) -> int:
+        return sum(g * (dk + dv) for g, dk, dv in self.kv_layer_shapes(0, layers)) * dtype_bytes
+
+    def param_count(self) -> int:
+        W = self.hidden_size
+        n = 2 * self.vocab_size * W
+        for l in self.layers:
+            m = l.mixer
+            n += W * (m.q_size + m.k_size + m.v_size + m.o_size) + m.o_size * W
+            if l.mlp is not None:
+                n += 3 * W * l.mlp.ff
+        return n
+
+    def to_dict(self) -> dict:
+        return dataclasses.asdict(self)
+
+    @staticmethod
+    def from_dict(d: dict, name: str = "bebovik") -> "BebovikConfig":
+        layers = []
+        for e in d["layers"]:
+            if e["type"] != "attention":
+                raise ValueError(f"Bebovik: unknown mixer type {e['type']!r}")
+            m = e["mixer"]
+            rot = m.get("rot")
+            mask = m.get("mask") or {}
+            spec = AttentionSpec(
+                heads=int(m["heads"]), kv_heads=int(m["kv_heads"]), dim=int(m["dim"]), vdim=int(m["vdim"]),
+                scale=float(m["scale"]),
+                rot=None if not rot else RotarySpec(float(rot["base"]), int(rot["dims"]), rot.get("scaling") or None),
+                mask_kind="chunk" if mask.get("size") else "causal", mask_size=int(mask.get("size") or 0))
+            if spec.heads % spec.kv_heads:
+                raise ValueError("Bebovik: heads must be a multiple of kv_heads")
+            f = e.get("mlp")
+            if f is not None and f.get("kind", "dense") != "dense":
+                raise ValueError(f"Bebovik: unknown feed-forward kind {f.get('kind')!r}")
+            layers.append(LayerSpec(e["type"], spec, None if f is None else GluSpec(int(f["ff"]), float(f["limit"]))))
+        return BebovikConfig(name=name, vocab_size=int(d["vocab"]), hidden_size=int(d["width"]), layers=layers,
+                             embedding_scale=float(d.get("embedding", {}).get("scale", 1.0)),
+                             logit_scale=float(d.get("logit_scale", 1.0)),
+                             logit_softcap=float(d.get("logit_softcap") or 0.0),
+                             norm_eps=float(d.get("norm", {}).get("eps", 1e-6)))
+
+
+def bebovik_uniform(name: str, vocab: int, width: int, n_layers: int, heads: int, kv_heads: int, dim: int,
+                    vdim: int, ff: int, chunk: int, rot_dims: Optional[int] = None, base: float = 10000.0,
+                    scaling: Optional[dict] = None, limit: float = 7.0, **kw) -> BebovikConfig:
+    """A Bebovik configuration whose layers all share one geometry (presets, benchmarks)."""
+    def layer():
+        return LayerSpec("attention", AttentionSpec(heads, kv_heads, dim, vdim, dim ** -0.5,
+                                                    RotarySpec(base, rot_dims or dim, scaling),
+                                                    "chunk" if chunk else "causal", chunk),
+                         GluSpec(ff, limit) if ff else None)
+    return BebovikConfig(name=name, vocab_size=vocab, hidden_size=width, layers=[layer() for _ in range(n_layers)], **kw)
+
+
+NATIVE_CONFIGS = {"bebovik": BebovikConfig.from_dict}
 
 
 PRESETS: dict[str, ModelConfig] = {
@@ -153,6 +321,10 @@ PRESETS: dict[str, ModelConfig] = {
                             num_layers=2, num_heads=8, num_kv_heads=2, head_dim=128, rope_theta=10000.0,
                             rms_eps=1.5625e-07, max_position=4096, qkv_bias=True, rotary_dim=64,
                             rope_interleaved=True, bos_token_id=1, eos_token_id=2),
+    # Bebovik test / smoke sizes (random weights): chunk-masked GQA attention, half-rotary heads
+    "bebovik-tiny": bebovik_uniform("bebovik-tiny", 1024, 256, 3, 4, 2, 64, 64, 512, 48, rot_dims=32,
+                                    embedding_scale=4.0, logit_scale=0.5, logit_softcap=30.0, max_position=4096,
+                                    bos_token_id=1, eos_token_id=2),
     "opt-125m": ModelConfig(name="opt-125m", arch="opt", vocab_size=50272, hidden_size=768,
                             intermediate_size=3072, num_layers=12, num_heads=12, num_kv_heads=12, head_dim=64,
                             max_position=2048, tie_embeddings=True, bos_token_id=2, eos_token_id=2),
@@ -181,10 +353,14 @@ def get_config(name_or_path: str) -> ModelConfig:
     (multi-rank rehearsals of a big model's shapes on one GPU)."""
     if "@L" in name_or_path:
         base, n = name_or_path.rsplit("@L", 1)
-        return dataclasses.replace(get_config(base), name=name_or_path, num_layers=int(n))
+        bc = get_config(base)
+        if isinstance(bc, BebovikConfig):
+            return dataclasses.replace(bc, name=name_or_path, layers=bc.layers[: int(n)])
+        return dataclasses.replace(bc, name=name_or_path, num_layers=int(n))
     key = ALIASES.get(name_or_path, name_or_path)
     if key in PRESETS:
-        return dataclasses.replace(PRESETS[key])
+        import copy
+        return copy.deepcopy(PRESETS[key])
     if os.path.exists(name_or_path):
         return ModelConfig.from_file(name_or_path)
     lk = key.lower()

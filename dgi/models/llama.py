@@ -330,6 +330,10 @@ class LlamaModel:
             n += self.lm_head.numel() * self.lm_head.element_size()
         return n
 
+    def attach_cache(self, pool) -> None:
+        """Bind the engine's block pool (one [L, 2, NB, n_kv, bs, hd] tensor)."""
+        self.kv_cache = pool.kv
+
     # ------------------------------------------------------------------ forward
     def attention(self, li: int, qkv: torch.Tensor, meta: AttnMeta, rope: bool = True,
                   out: Optional[torch.Tensor] = None) -> torch.Tensor:

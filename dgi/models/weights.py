@@ -93,7 +93,7 @@ class CheckpointReader:
         """Tensor ``name`` (optionally rows [a, b) / cols [a, b) only) as a CPU tensor."""
         sl = self._h(name).get_slice(name)
         if rows is None and cols is None:
-            t = sl[:]
+            t = sl[:] if len(sl.get_shape()) else self._h(name).get_tensor(name)     # 0-dim: no slicing
         elif cols is None:
             t = sl[rows[0]:rows[1]]
         elif rows is None:
@@ -167,6 +167,60 @@ def load_checkpoint(model, path: str, tp_rank: int = 0, tp: int = 1) -> dict:
             else:   # tied checkpoint served by an untied slot (last stage without the embedding)
                 _put(model.lm_head, rd.read("model.embed_tokens.weight"))
             n += 1
+    out = {"tensors": n, "bytes": rd.bytes_read, "path": path}
+    rd.close()
+    return out
+
+
+def load_bebovik_checkpoint(model, path: str) -> dict:
+    """Fill a ``BebovikModel`` from the design's safetensors layout: ``embed`` / ``head``,
+    norms as ``<name>`` (weight), ``<name>.b`` and the scalar ``<name>.alpha``, and per layer i
+    ``l<i>.mix.{q,k,v,g,o}`` (stored [out, in]), ``l<i>.mix.{q,k}.norm``, ``l<i>.mlp.{gate,up,down}``,
+    ``l<i>.ls1`` / ``ls2``.  q | k | v | g land in the fused projection weight and gate | up in the
+    fused feed-forward weight; only the model's own layer range is read.  Norm parameters,
+    layer scales and q/k norm weights are kept in fp32."""
+    rd = CheckpointReader(path)
+    n = 0
+
+    def put(dst, name):
+        nonlocal n
+        src = rd.read(name)
+        _put(dst, src.reshape(dst.shape) if src.numel() == dst.numel() and src.dim() != dst.dim() else src)
+        n += 1
+
+    def put_norm(norm, name):
+        put(norm.w, name)
+        put(norm.b, name + ".b")
+        put(norm.alpha, name + ".alpha")
+
+    for i, li in enumerate(range(model.layer_start, model.layer_end)):
+        L = model.layers[i]
+        m = L.spec.mixer
+        p = f"l{li}."
+        r = 0
+        for key, rows in (("q", m.q_size), ("k", m.k_size), ("v", m.v_size), ("g", m.o_size)):
+            put(L.qkvg[r:r + rows], p + "mix." + key)
+            r += rows
+        put(L.o, p + "mix.o")
+        put(L.q_norm, p + "mix.q.norm")
+        put(L.k_norm, p + "mix.k.norm")
+        put_norm(L.norm1, p + "norm1")
+        put_norm(L.norm1b, p + "norm1b")
+        put(L.ls1, p + "ls1")
+        if L.gate_up is not None:
+            ff = L.spec.mlp.ff
+            put(L.gate_up[:ff], p + "mlp.gate")
+            put(L.gate_up[ff:], p + "mlp.up")
+            put(L.down, p + "mlp.down")
+            put_norm(L.norm2, p + "norm2")
+            put_norm(L.norm2b, p + "norm2b")
+            put(L.ls2, p + "ls2")
+    if model.embed is not None:
+        put(model.embed, "embed")
+        put_norm(model.embed_norm, "embed.norm")
+    if model.has_head:
+        put(model.head, "head")
+        put_norm(model.final_norm, "final.norm")
     out = {"tensors": n, "bytes": rd.bytes_read, "path": path}
     rd.close()
     return out

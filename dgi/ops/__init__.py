@@ -122,11 +122,12 @@ def rope_cos_sin(head_dim: int, max_pos: int, theta: float, scaling: Optional[di
     Supports Llama-3.1 style ``rope_scaling`` (``rope_type == "llama3"``).
     """
     inv = 1.0 / (theta ** (torch.arange(0, head_dim, 2, dtype=torch.float64) / head_dim))
-    if scaling and scaling.get("rope_type", scaling.get("type")) == "llama3":
+    if scaling and (scaling.get("rope_type", scaling.get("type")) == "llama3" or "original" in scaling):
+        # wavelength-dependent rescale; HF key names, or the short ones (factor, low, high, original)
         factor = scaling["factor"]
-        lo = scaling.get("low_freq_factor", 1.0)
-        hi = scaling.get("high_freq_factor", 4.0)
-        old = scaling.get("original_max_position_embeddings", 8192)
+        lo = scaling.get("low_freq_factor", scaling.get("low", 1.0))
+        hi = scaling.get("high_freq_factor", scaling.get("high", 4.0))
+        old = scaling.get("original_max_position_embeddings", scaling.get("original", 8192))
         lo_wl, hi_wl = old / lo, old / hi
         wl = 2 * math.pi / inv
         smooth = (old / wl - lo) / (hi - lo)
@@ -367,6 +368,11 @@ def paged_prefill(q, k_cache, v_cache, block_tables, cu_seqlens_q, context_lens,
         out.copy_(r)
         return out
     return r
+
+
+def masked_prefill_available() -> bool:
+    """Whether the MFMA prompt-attention kernel with a block mask and gate epilogue is built."""
+    return False
 
 
 # ----------------------------------------------------------------------------

@@ -1,0 +1,243 @@
+"""Mixer-block ops for models with fp32 residual streams and per-layer head geometry
+(``dgi/_C_mix.so``, sources in ``dgi/csrc/mix``): Dynamic-Tanh norms, per-head q/k RMS norm +
+interleaved rotary + paged KV write, row-wise masked attention, clamped GLU, soft-capped logits.
+
+Same contract as the rest of ``dgi.ops``: the HIP kernel runs whenever the tensors are on the
+GPU (and raises if the library is missing), the ``*_ref`` function — plain PyTorch, fp32 math —
+runs on CPU tensors and is the oracle of the kernel tests.  Activations are bf16 or fp32; norm
+parameters and the residual stream are fp32 in both.
+"""
+from __future__ import annotations
+
+import os
+from typing import Optional
+
+import torch
+
+_LIB = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "_C_mix.so")
+_loaded = False
+
+
+def load_native(required: bool = False) -> bool:
+    """Load ``dgi/_C_mix.so`` once (built by ``python -m dgi.build mix``)."""
+    global _loaded
+    if _loaded:
+        return True
+    err = f"{_LIB} not built (run `python -m dgi.build mix`)"
+    if os.path.exists(_LIB):
+        try:
+            torch.ops.load_library(_LIB)
+            _loaded = True
+            return True
+        except Exception as e:  # pragma: no cover - depends on the box
+            err = repr(e)
+    if required:
+        raise RuntimeError(f"dgi mixer kernels unavailable: {err}")
+    return False
+
+
+def _native(t: torch.Tensor) -> bool:
+    if t.is_cuda:
+        load_native(required=True)
+        return True
+    return False
+
+
+def _call(name: str, *args) -> None:
+    from dgi import ops
+    getattr(torch.ops.dgi, name)(*args)
+    if ops._DEBUG_SYNC:
+        from dgi.utils.debug import after_op
+        after_op(name, *args)
+
+
+class DytNorm:
+    """Parameters of one Dynamic-Tanh norm, y = tanh(alpha * x) * w + b (all fp32)."""
+    __slots__ = ("alpha", "w", "b")
+
+    def __init__(self, alpha: torch.Tensor, w: torch.Tensor, b: torch.Tensor):
+        self.alpha, self.w, self.b = alpha, w, b
+
+    def tensors(self):
+        return (("alpha", self.alpha), ("w", self.w), ("b", self.b))
+
+
+# ----------------------------------------------------------------------------
+# Dynamic-Tanh norms
+# ----------------------------------------------------------------------------
+
+def dyt_ref(x: torch.Tensor, n: DytNorm, dtype: torch.dtype) -> torch.Tensor:
+    return (torch.tanh(n.alpha * x.float()) * n.w + n.b).to(dtype)
+
+
+def dyt(x: torch.Tensor, n: DytNorm, dtype: torch.dtype) -> torch.Tensor:
+    """Norm of the fp32 stream ``x`` [T, W] -> [T, W] in ``dtype`` (the GEMM input)."""
+    if _native(x):
+        y = torch.empty(x.shape, dtype=dtype, device=x.device)
+        _call("dyt", y, x, n.alpha, n.w, n.b)
+        return y
+    return dyt_ref(x, n, dtype)
+
+
+def dyt_add_ref(res: torch.Tensor, h: torch.Tensor, post: DytNorm, ls: torch.Tensor,
+                nxt: Optional[DytNorm] = None) -> Optional[torch.Tensor]:
+    res.add_((torch.tanh(post.alpha * h.float()) * post.w + post.b) * ls)
+    return None if nxt is None else dyt_ref(res, nxt, h.dtype)
+
+
+def dyt_add(res: torch.Tensor, h: torch.Tensor, post: DytNorm, ls: torch.Tensor,
+            nxt: Optional[DytNorm] = None) -> Optional[torch.Tensor]:
+    """res += post(h) * ls in place (sublayer output norm, layer scale, residual add); with
+    ``nxt`` also returns nxt(res) in h's dtype — the next sublayer's input, from the same pass."""
+    if _native(res):
+        y = torch.empty(res.shape, dtype=h.dtype, device=res.device) if nxt is not None else None
+        _call("dyt_add", res, h, post.alpha, post.w, post.b, ls, y, *((nxt.alpha, nxt.w, nxt.b) if nxt else (None,) * 3))
+        return y
+    return dyt_add_ref(res, h, post, ls, nxt)
+
+
+def embed_dyt_ref(ids: torch.Tensor, table: torch.Tensor, scale: float, n: DytNorm) -> torch.Tensor:
+    return dyt_ref(table[ids.long()].float() * scale, n, torch.float32)
+
+
+def embed_dyt(ids: torch.Tensor, table: torch.Tensor, scale: float, n: DytNorm) -> torch.Tensor:
+    """fp32 stream [T, W] = n(table[ids] * scale)."""
+    if _native(table):
+        res = torch.empty(ids.numel(), table.shape[1], dtype=torch.float32, device=table.device)
+        _call("embed_dyt", res, ids.long().contiguous(), table, float(scale), n.alpha, n.w, n.b)
+        return res
+    return embed_dyt_ref(ids, table, scale, n)
+
+
+# ----------------------------------------------------------------------------
+# q/k norm + rotary + paged cache write
+# ----------------------------------------------------------------------------
+
+def _rot_pairs(x: torch.Tensor, cs: torch.Tensor) -> torch.Tensor:
+    """Interleaved-pair rotation of the first rd = cs.shape[-1] dims of x [T, heads, d] (fp32)."""
+    rd = cs.shape[-1]
+    if rd == 0:
+        return x
+    c, s = cs[:, None, : rd // 2], cs[:, None, rd // 2:]
+    u, v = x[..., 0:rd:2], x[..., 1:rd:2]
+    r = torch.stack([u * c - v * s, v * c + u * s], dim=-1).flatten(-2)
+    return torch.cat([r, x[..., rd:]], dim=-1)
+
+
+def qknorm_rope_cache_ref(qkv, positions, slots, qw, kw, eps, cos_sin, H, G, dk, dv, k_cache, v_cache) -> None:
+    T = qkv.shape[0]
+    if T == 0:
+        return
+    bs = k_cache.shape[2]
+    q = qkv[:, : H * dk].float().view(T, H, dk)
+    k = qkv[:, H * dk:(H + G) * dk].float().view(T, G, dk)
+    v = qkv[:, (H + G) * dk:(H + G) * dk + G * dv].view(T, G, dv)
+    q = q / torch.sqrt(q.pow(2).mean(-1, keepdim=True) + eps) * qw
+    k = k / torch.sqrt(k.pow(2).mean(-1, keepdim=True) + eps) * kw
+    if cos_sin is not None:
+        cs = cos_sin[positions.long()]
+        q, k = _rot_pairs(q, cs), _rot_pairs(k, cs)
+    qkv[:, : H * dk] = q.reshape(T, H * dk).to(qkv.dtype)
+    ok = slots >= 0
+    if ok.any():
+        s = slots[ok].long()
+        k_cache[s // bs, :, s % bs] = k[ok].to(k_cache.dtype)
+        v_cache[s // bs, :, s % bs] = v[ok]
+
+
+def qknorm_rope_cache(qkv, positions, slots, qw, kw, eps: float, cos_sin, H: int, G: int, dk: int, dv: int,
+                      k_cache, v_cache) -> None:
+    """Rows of ``qkv`` = [q: H*dk | k: G*dk | v: G*dv | ...]: per-head RMS norm (weights ``qw`` /
+    ``kw`` [dk], eps inside the root) and interleaved rotary (``cos_sin`` [max_pos, rd], or None)
+    of q in place and of k into ``k_cache`` [NB, G, bs, dk]; v into ``v_cache`` [NB, G, bs, dv]
+    at ``slots`` (-1: not written)."""
+    if _native(qkv):
+        _call("qknorm_rope_cache", qkv, positions, slots, qw, kw, float(eps), cos_sin, H, G, dk, dv, k_cache, v_cache)
+    else:
+        qknorm_rope_cache_ref(qkv, positions, slots, qw, kw, eps, cos_sin, H, G, dk, dv, k_cache, v_cache)
+
+
+# ----------------------------------------------------------------------------
+# Row-wise masked attention
+# ----------------------------------------------------------------------------
+
+def masked_attn_rows_ref(q, k_cache, v_cache, block_tables, cu_seqlens, positions, H, G, scale, mask, gate=None):
+    T = q.shape[0]
+    bs, dk, dv = k_cache.shape[2], k_cache.shape[3], v_cache.shape[3]
+    out = torch.zeros(T, H * dv, dtype=q.dtype, device=q.device)
+    cu = cu_seqlens.tolist() if cu_seqlens is not None else None
+    pos = positions.tolist()
+    seq = 0
+    for t in range(T):
+        if cu is None:
+            seq = t
+        else:
+            while cu[seq + 1] <= t:
+                seq += 1
+        p = pos[t]
+        first = (p // mask) * mask if mask > 0 else 0
+        keys = torch.arange(first, p + 1, device=q.device)
+        blk = block_tables[seq][keys // bs].long()
+        k = k_cache[blk, :, keys % bs].float()          # [n, G, dk]
+        v = v_cache[blk, :, keys % bs].float()
+        qt = q[t, : H * dk].float().view(G, H // G, dk)
+        s = torch.einsum("ghd,ngd->ghn", qt, k) * scale
+        o = torch.einsum("ghn,ngd->ghd", torch.softmax(s, dim=-1), v).reshape(H * dv)
+        if gate is not None:
+            o = o * torch.sigmoid(gate[t, : H * dv].float())
+        out[t] = o.to(q.dtype)
+    return out
+
+
+def masked_attn_rows(q, k_cache, v_cache, block_tables, cu_seqlens, positions, H: int, G: int, scale: float,
+                     mask: int = 0, gate=None, out=None) -> torch.Tensor:
+    """Softmax attention of each row of ``q`` (position ``positions[t]``) over keys
+    [floor(p / mask) * mask, p] of its sequence (``mask`` 0: [0, p]) read from the paged cache;
+    rows map to ``block_tables`` rows through ``cu_seqlens`` (None: row i <-> table row i).
+    ``gate``: the output is multiplied by sigmoid(gate) element by element."""
+    if _native(q):
+        if out is None:
+            out = torch.empty(q.shape[0], H * v_cache.shape[3], dtype=q.dtype, device=q.device)
+        _call("masked_attn_rows", out, q, k_cache, v_cache, block_tables, cu_seqlens, positions, H, G, float(scale),
+              int(mask), gate)
+        return out
+    r = masked_attn_rows_ref(q, k_cache, v_cache, block_tables, cu_seqlens, positions, H, G, scale, mask, gate)
+    if out is not None:
+        out.copy_(r)
+        return out
+    return r
+
+
+# ----------------------------------------------------------------------------
+# Activations / logits
+# ----------------------------------------------------------------------------
+
+def glu_clamped_ref(gu: torch.Tensor, limit: float, alpha: float = 1.702) -> torch.Tensor:
+    I = gu.shape[-1] // 2
+    g = gu[..., :I].float().clamp(max=limit)
+    u = gu[..., I:].float().clamp(-limit, limit)
+    return (g * torch.sigmoid(alpha * g) * (u + 1.0)).to(gu.dtype)
+
+
+def glu_clamped(gu: torch.Tensor, limit: float, alpha: float = 1.702) -> torch.Tensor:
+    """g * sigmoid(alpha g) * (u + 1) over the fused [gate | up] rows, gate clamped from above
+    and up to [-limit, limit]."""
+    if _native(gu):
+        out = torch.empty(gu.shape[0], gu.shape[1] // 2, dtype=gu.dtype, device=gu.device)
+        _call("glu_clamped", out, gu, float(limit), float(alpha))
+        return out
+    return glu_clamped_ref(gu, limit, alpha)
+
+
+def scale_softcap_ref(x: torch.Tensor, scale: float, cap: float) -> torch.Tensor:
+    v = x.float() * scale
+    return cap * torch.tanh(v / cap) if cap > 0 else v
+
+
+def scale_softcap(x: torch.Tensor, scale: float, cap: float) -> torch.Tensor:
+    """fp32 logits = cap * tanh(x * scale / cap) (cap <= 0: x * scale)."""
+    if _native(x):
+        out = torch.empty(x.shape, dtype=torch.float32, device=x.device)
+        _call("scale_softcap", out, x, float(scale), float(cap))
+        return out
+    return scale_softcap_ref(x, scale, cap)

@@ -115,7 +115,10 @@ class ModelRunner:
         self.max_tokens = max_num_batched_tokens
         self.num_cus = num_cus
         self.step_id = 0
-        model.kv_cache = pool.kv
+        if hasattr(model, "attach_cache"):
+            model.attach_cache(pool)
+        else:
+            model.kv_cache = pool.kv
         self.is_cuda = self.device.type == "cuda"
         # decode split-KV plan used by graphs (fixed) and workspaces
         self.graph_part = decode_part_size
@@ -218,7 +221,10 @@ class ModelRunner:
             pre_bt[j, : len(r.blocks)] = blk
             cu[j + 1] = cu[j] + c.length
             pctx[j] = c.start + c.length
-            if c.sample:
+            if c.logit_pos is not None:     # replay: logits of the given offsets, nothing sampled
+                logit_rows.extend(row + p for p in c.logit_pos)
+                sampled.extend([r] * len(c.logit_pos))
+            elif c.sample:
                 logit_rows.append(row + c.length - 1)
                 sampled.append(r)
             row += c.length
@@ -311,6 +317,17 @@ class ModelRunner:
         toks = samp.sample(logits)
         self._span_end(span)
         return StepResult(self.fetch(toks), sampled)
+
+    @torch.inference_mode()
+    def execute_logits(self, sb: ScheduledBatch) -> torch.Tensor:
+        """One eager step that samples nothing: the fp32 logits of the step's logits rows (every
+        decode row, then each chunk's ``logit_pos`` rows or sampled last row), on the host."""
+        self.step_id += 1
+        self.gate_rows(sb.decode, sb.prefill)
+        flat, hdr, _sampled = self.build_host(sb)
+        ids, meta, _samp = self.meta_from_device(self.to_device(flat), hdr)
+        logits = self.model.forward(meta, input_ids=ids)
+        return logits.float().cpu()
 
     # DGI_GPU_SPAN=1: events around each eager step's device work (forward + sampling);
     # wall time minus the summed spans is the time the GPU waited for the host

@@ -56,6 +56,9 @@ class PrefillChunk:
     start: int       # first token index of the chunk (== req.num_computed)
     length: int
     sample: bool     # chunk completes the prefill target -> sample a token
+    # offsets inside the chunk whose logits the step also returns (teacher-forced replay,
+    # ``LLMEngine.feed``); None: only the sampled last row
+    logit_pos: Optional[list] = None
 
 
 @dataclasses.dataclass
