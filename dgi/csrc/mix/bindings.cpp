@@ -24,6 +24,10 @@ int dgi_masked_attn_rows(const void* q, int q_stride, const void* k_cache, const
                          int bt_stride, const int* cu_seqlens, int n_seqs, const int* positions, int rows, int H, int G,
                          int dk, int dv, int block_size, float scale, int mask, const void* gate, int gate_stride,
                          void* out, int out_stride, int is_f32, hipStream_t s);
+int dgi_paged_prefill_masked(const void* q, int q_stride, const void* k_cache, const void* v_cache,
+                             const int* block_tables, int bt_stride, const int* cu_seqlens_q, const int* context_lens,
+                             const int* tiles, int n_tiles, void* out, int out_stride, int nh, int nkv, int hd,
+                             int block_size, float scale, int mask, const void* gate, int gate_stride, hipStream_t s);
 int dgi_glu_clamped(const void* gu, int gu_stride, void* out, int is_f32, int T, int I, float limit, float alpha,
                     hipStream_t s);
 int dgi_scale_softcap(const void* x, int x_stride, float* out, int is_f32, int T, int V, float scale, float cap,
@@ -168,6 +172,42 @@ void masked_attn_rows(at::Tensor out, const at::Tensor& q, const at::Tensor& k_c
            "masked_attn_rows");
 }
 
+// bf16, key size == value size in {64, 128}: packed prompt portions (cu_seqlens_q) over
+// [cached prefix | new keys]; tiles [n, 2] = (sequence, first row of a 128-row tile)
+void paged_prefill_masked(at::Tensor out, const at::Tensor& q, const at::Tensor& k_cache, const at::Tensor& v_cache,
+                          const at::Tensor& block_tables, const at::Tensor& cu_seqlens_q, const at::Tensor& context_lens,
+                          const at::Tensor& tiles, int64_t nh, int64_t nkv, double scale, int64_t mask,
+                          const c10::optional<at::Tensor>& gate) {
+  TORCH_CHECK(act_kind(q, "q") == 0 && act_kind(out, "out") == 0 && act_kind(k_cache, "k_cache") == 0 &&
+              act_kind(v_cache, "v_cache") == 0, "paged_prefill_masked: bfloat16 only");
+  check_rows(q, "q"); check_rows(out, "out");
+  check_i32(block_tables, "block_tables"); check_i32(cu_seqlens_q, "cu_seqlens_q");
+  check_i32(context_lens, "context_lens"); check_i32(tiles, "tiles");
+  TORCH_CHECK(k_cache.is_contiguous() && v_cache.is_contiguous() && k_cache.dim() == 4 && k_cache.sizes() == v_cache.sizes());
+  const int hd = (int)k_cache.size(3);
+  TORCH_CHECK(k_cache.size(1) == nkv && q.size(1) >= nh * hd && out.size(1) >= nh * hd && out.size(0) == q.size(0));
+  TORCH_CHECK(q.stride(0) % 8 == 0 && out.stride(0) % 4 == 0 && q.data_ptr<at::BFloat16>() != nullptr);
+  TORCH_CHECK(reinterpret_cast<uintptr_t>(q.data_ptr()) % 16 == 0 && reinterpret_cast<uintptr_t>(out.data_ptr()) % 8 == 0,
+              "paged_prefill_masked: q must be 16-byte and out 8-byte aligned");
+  const int nb = (int)cu_seqlens_q.numel() - 1;
+  TORCH_CHECK(block_tables.dim() == 2 && block_tables.size(0) >= nb && context_lens.numel() >= nb);
+  TORCH_CHECK(tiles.dim() == 2 && tiles.size(1) == 2);
+  const void* gp = nullptr;
+  int gs = 0;
+  if (gate.has_value()) {
+    check_rows(*gate, "gate");
+    TORCH_CHECK(act_kind(*gate, "gate") == 0 && gate->size(0) == q.size(0) && gate->size(1) >= nh * hd);
+    TORCH_CHECK(gate->stride(0) % 4 == 0 && reinterpret_cast<uintptr_t>(gate->data_ptr()) % 8 == 0, "gate alignment");
+    gp = gate->data_ptr();
+    gs = (int)gate->stride(0);
+  }
+  check_rc(dgi_paged_prefill_masked(q.data_ptr(), (int)q.stride(0), k_cache.data_ptr(), v_cache.data_ptr(),
+                                    block_tables.data_ptr<int>(), (int)block_tables.stride(0), cu_seqlens_q.data_ptr<int>(),
+                                    context_lens.data_ptr<int>(), tiles.data_ptr<int>(), (int)tiles.size(0), out.data_ptr(),
+                                    (int)out.stride(0), (int)nh, (int)nkv, hd, (int)k_cache.size(2), (float)scale, (int)mask,
+                                    gp, gs, cur_stream()), "paged_prefill_masked");
+}
+
 void glu_clamped(at::Tensor out, const at::Tensor& gu, double limit, double alpha) {
   const int f = act_kind(gu, "gu");
   check_rows(gu, "gu");
@@ -196,6 +236,9 @@ TORCH_LIBRARY_FRAGMENT(dgi, m) {
         "Tensor? cos_sin, int H, int G, int dk, int dv, Tensor(b!) k_cache, Tensor(c!) v_cache) -> ()");
   m.def("masked_attn_rows(Tensor(a!) out, Tensor q, Tensor k_cache, Tensor v_cache, Tensor block_tables, "
         "Tensor? cu_seqlens, Tensor positions, int H, int G, float scale, int mask, Tensor? gate) -> ()");
+  m.def("paged_prefill_masked(Tensor(a!) out, Tensor q, Tensor k_cache, Tensor v_cache, Tensor block_tables, "
+        "Tensor cu_seqlens_q, Tensor context_lens, Tensor tiles, int nh, int nkv, float scale, int mask, "
+        "Tensor? gate) -> ()");
   m.def("glu_clamped(Tensor(a!) out, Tensor gu, float limit, float alpha) -> ()");
   m.def("scale_softcap(Tensor(a!) out, Tensor x, float scale, float cap) -> ()");
 }
@@ -206,6 +249,7 @@ TORCH_LIBRARY_IMPL(dgi, CUDA, m) {
   m.impl("embed_dyt", &embed_dyt);
   m.impl("qknorm_rope_cache", &qknorm_rope_cache);
   m.impl("masked_attn_rows", &masked_attn_rows);
+  m.impl("paged_prefill_masked", &paged_prefill_masked);
   m.impl("glu_clamped", &glu_clamped);
   m.impl("scale_softcap", &scale_softcap);
 }
