@@ -33,16 +33,48 @@ struct DytParams {
   const float* b;       // [W]
 };
 
-template <typename TA>
+// four consecutive elements per thread (W % 4 == 0: 16-byte fp32 / 8-byte bf16 accesses)
+template <typename T> __device__ __forceinline__ void ld4(const T* p, float* f);
+template <> __device__ __forceinline__ void ld4<float>(const float* p, float* f) {
+  const float4 v = *reinterpret_cast<const float4*>(p);
+  f[0] = v.x; f[1] = v.y; f[2] = v.z; f[3] = v.w;
+}
+template <> __device__ __forceinline__ void ld4<uint16_t>(const uint16_t* p, float* f) {
+  const uint2 v = *reinterpret_cast<const uint2*>(p);
+  f[0] = __uint_as_float(v.x << 16); f[1] = __uint_as_float(v.x & 0xffff0000u);
+  f[2] = __uint_as_float(v.y << 16); f[3] = __uint_as_float(v.y & 0xffff0000u);
+}
+template <typename T> __device__ __forceinline__ void st4(T* p, const float* f);
+template <> __device__ __forceinline__ void st4<float>(float* p, const float* f) {
+  *reinterpret_cast<float4*>(p) = make_float4(f[0], f[1], f[2], f[3]);
+}
+template <> __device__ __forceinline__ void st4<uint16_t>(uint16_t* p, const float* f) {
+  uint2 v;
+  v.x = pack_bf16x2(f[0], f[1]);
+  v.y = pack_bf16x2(f[2], f[3]);
+  *reinterpret_cast<uint2*>(p) = v;
+}
+
+template <typename TA, bool VEC>
 __global__ __launch_bounds__(256) void dyt_kernel(const float* __restrict__ x, DytParams n, TA* __restrict__ y,
                                                   int W) {
   const size_t row = (size_t)blockIdx.x * W;
   const float a = n.alpha[0];
-  for (int c = threadIdx.x; c < W; c += 256) stf<TA>(y + row + c, tanhf(a * x[row + c]) * n.w[c] + n.b[c]);
+  if (VEC) {
+    for (int c = threadIdx.x * 4; c < W; c += 1024) {
+      float v[4], w[4], b[4], o[4];
+      ld4<float>(x + row + c, v); ld4<float>(n.w + c, w); ld4<float>(n.b + c, b);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) o[j] = tanhf(a * v[j]) * w[j] + b[j];
+      st4<TA>(y + row + c, o);
+    }
+  } else {
+    for (int c = threadIdx.x; c < W; c += 256) stf<TA>(y + row + c, tanhf(a * x[row + c]) * n.w[c] + n.b[c]);
+  }
 }
 
 // res += (tanh(a1 * h) * w1 + b1) * ls;  y = tanh(a2 * res) * w2 + b2 (when y != nullptr)
-template <typename TA>
+template <typename TA, bool VEC>
 __global__ __launch_bounds__(256) void dyt_add_kernel(const TA* __restrict__ h, int h_stride, DytParams post,
                                                       const float* __restrict__ ls, float* __restrict__ res,
                                                       DytParams next, TA* __restrict__ y, int W) {
@@ -50,14 +82,32 @@ __global__ __launch_bounds__(256) void dyt_add_kernel(const TA* __restrict__ h, 
   const TA* hr = h + (size_t)blockIdx.x * h_stride;
   const float a1 = post.alpha[0];
   const float a2 = y ? next.alpha[0] : 0.f;
-  for (int c = threadIdx.x; c < W; c += 256) {
-    const float v = res[row + c] + (tanhf(a1 * ldf<TA>(hr + c)) * post.w[c] + post.b[c]) * ls[c];
-    res[row + c] = v;
-    if (y) stf<TA>(y + row + c, tanhf(a2 * v) * next.w[c] + next.b[c]);
+  if (VEC) {
+    for (int c = threadIdx.x * 4; c < W; c += 1024) {
+      float hv[4], r[4], w[4], b[4], l[4];
+      ld4<TA>(hr + c, hv); ld4<float>(res + row + c, r);
+      ld4<float>(post.w + c, w); ld4<float>(post.b + c, b); ld4<float>(ls + c, l);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) r[j] += (tanhf(a1 * hv[j]) * w[j] + b[j]) * l[j];
+      st4<float>(res + row + c, r);
+      if (y) {
+        float o[4];
+        ld4<float>(next.w + c, w); ld4<float>(next.b + c, b);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) o[j] = tanhf(a2 * r[j]) * w[j] + b[j];
+        st4<TA>(y + row + c, o);
+      }
+    }
+  } else {
+    for (int c = threadIdx.x; c < W; c += 256) {
+      const float v = res[row + c] + (tanhf(a1 * ldf<TA>(hr + c)) * post.w[c] + post.b[c]) * ls[c];
+      res[row + c] = v;
+      if (y) stf<TA>(y + row + c, tanhf(a2 * v) * next.w[c] + next.b[c]);
+    }
   }
 }
 
-template <typename TA>
+template <typename TA, bool VEC>
 __global__ __launch_bounds__(256) void embed_dyt_kernel(const long long* __restrict__ ids, const TA* __restrict__ table,
                                                         int vocab, float scale, DytParams n, float* __restrict__ res,
                                                         int W) {
@@ -66,7 +116,17 @@ __global__ __launch_bounds__(256) void embed_dyt_kernel(const long long* __restr
   id = id < 0 ? 0 : (id >= vocab ? vocab - 1 : id);
   const TA* e = table + (size_t)id * W;
   const float a = n.alpha[0];
-  for (int c = threadIdx.x; c < W; c += 256) res[row + c] = tanhf(a * (ldf<TA>(e + c) * scale)) * n.w[c] + n.b[c];
+  if (VEC) {
+    for (int c = threadIdx.x * 4; c < W; c += 1024) {
+      float v[4], w[4], b[4], o[4];
+      ld4<TA>(e + c, v); ld4<float>(n.w + c, w); ld4<float>(n.b + c, b);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) o[j] = tanhf(a * (v[j] * scale)) * w[j] + b[j];
+      st4<float>(res + row + c, o);
+    }
+  } else {
+    for (int c = threadIdx.x; c < W; c += 256) res[row + c] = tanhf(a * (ldf<TA>(e + c) * scale)) * n.w[c] + n.b[c];
+  }
 }
 
 }  // namespace
@@ -75,8 +135,14 @@ extern "C" int dgi_dyt(const float* x, const float* alpha, const float* w, const
                        int T, int W, hipStream_t s) {
   if (T == 0) return 0;
   const DytParams n{alpha, w, b};
-  if (is_f32) dyt_kernel<float><<<T, 256, 0, s>>>(x, n, (float*)y, W);
-  else dyt_kernel<uint16_t><<<T, 256, 0, s>>>(x, n, (uint16_t*)y, W);
+  const bool vec = W % 4 == 0 && ((uintptr_t)x | (uintptr_t)w | (uintptr_t)b | (uintptr_t)y) % 16 == 0;
+  if (is_f32) {
+    if (vec) dyt_kernel<float, true><<<T, 256, 0, s>>>(x, n, (float*)y, W);
+    else dyt_kernel<float, false><<<T, 256, 0, s>>>(x, n, (float*)y, W);
+  } else {
+    if (vec) dyt_kernel<uint16_t, true><<<T, 256, 0, s>>>(x, n, (uint16_t*)y, W);
+    else dyt_kernel<uint16_t, false><<<T, 256, 0, s>>>(x, n, (uint16_t*)y, W);
+  }
   DGI_CHECK_LAUNCH();
   return 0;
 }
@@ -86,10 +152,16 @@ extern "C" int dgi_dyt_add(const void* h, int h_stride, const float* alpha1, con
                            void* y, int is_f32, int T, int W, hipStream_t s) {
   if (T == 0) return 0;
   const DytParams post{alpha1, w1, b1}, next{alpha2, w2, b2};
-  if (is_f32)
-    dyt_add_kernel<float><<<T, 256, 0, s>>>((const float*)h, h_stride, post, ls, res, next, (float*)y, W);
-  else
-    dyt_add_kernel<uint16_t><<<T, 256, 0, s>>>((const uint16_t*)h, h_stride, post, ls, res, next, (uint16_t*)y, W);
+  const bool vec = W % 4 == 0 && h_stride % 4 == 0 &&
+                   ((uintptr_t)h | (uintptr_t)w1 | (uintptr_t)b1 | (uintptr_t)ls | (uintptr_t)res | (uintptr_t)w2 |
+                    (uintptr_t)b2 | (uintptr_t)y) % 16 == 0;
+  if (is_f32) {
+    if (vec) dyt_add_kernel<float, true><<<T, 256, 0, s>>>((const float*)h, h_stride, post, ls, res, next, (float*)y, W);
+    else dyt_add_kernel<float, false><<<T, 256, 0, s>>>((const float*)h, h_stride, post, ls, res, next, (float*)y, W);
+  } else {
+    if (vec) dyt_add_kernel<uint16_t, true><<<T, 256, 0, s>>>((const uint16_t*)h, h_stride, post, ls, res, next, (uint16_t*)y, W);
+    else dyt_add_kernel<uint16_t, false><<<T, 256, 0, s>>>((const uint16_t*)h, h_stride, post, ls, res, next, (uint16_t*)y, W);
+  }
   DGI_CHECK_LAUNCH();
   return 0;
 }
@@ -98,8 +170,14 @@ extern "C" int dgi_embed_dyt(const long long* ids, const void* table, int vocab,
                              const float* w, const float* b, float* res, int is_f32, int T, int W, hipStream_t s) {
   if (T == 0) return 0;
   const DytParams n{alpha, w, b};
-  if (is_f32) embed_dyt_kernel<float><<<T, 256, 0, s>>>(ids, (const float*)table, vocab, scale, n, res, W);
-  else embed_dyt_kernel<uint16_t><<<T, 256, 0, s>>>(ids, (const uint16_t*)table, vocab, scale, n, res, W);
+  const bool vec = W % 4 == 0 && ((uintptr_t)table | (uintptr_t)w | (uintptr_t)b | (uintptr_t)res) % 16 == 0;
+  if (is_f32) {
+    if (vec) embed_dyt_kernel<float, true><<<T, 256, 0, s>>>(ids, (const float*)table, vocab, scale, n, res, W);
+    else embed_dyt_kernel<float, false><<<T, 256, 0, s>>>(ids, (const float*)table, vocab, scale, n, res, W);
+  } else {
+    if (vec) embed_dyt_kernel<uint16_t, true><<<T, 256, 0, s>>>(ids, (const uint16_t*)table, vocab, scale, n, res, W);
+    else embed_dyt_kernel<uint16_t, false><<<T, 256, 0, s>>>(ids, (const uint16_t*)table, vocab, scale, n, res, W);
+  }
   DGI_CHECK_LAUNCH();
   return 0;
 }

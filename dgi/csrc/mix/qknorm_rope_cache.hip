@@ -11,7 +11,8 @@
 // The norm, its weight and the rotation are computed in fp32 whatever the activation dtype.
 //
 // Cache layout per layer: k [num_blocks, G, block_size, dk], v [num_blocks, G, block_size, dv].
-// One workgroup per token; a wave owns one head at a time (sum of squares by wave reduction).
+// One workgroup per token; a wave owns one head at a time (sum of squares by wave reduction),
+// a lane its rotation pairs; v rows are copied in 16-byte chunks where the sizes allow.
 #include "../common.h"
 
 using namespace dgi;
@@ -24,6 +25,23 @@ template <> __device__ __forceinline__ float ldf<uint16_t>(const uint16_t* p) { 
 template <typename T> __device__ __forceinline__ void stf(T* p, float v);
 template <> __device__ __forceinline__ void stf<float>(float* p, float v) { *p = v; }
 template <> __device__ __forceinline__ void stf<uint16_t>(uint16_t* p, float v) { *p = f32_to_bf16(v); }
+
+template <typename T> __device__ __forceinline__ void ld2(const T* p, float* f);
+template <> __device__ __forceinline__ void ld2<float>(const float* p, float* f) {
+  const float2 v = *reinterpret_cast<const float2*>(p);
+  f[0] = v.x; f[1] = v.y;
+}
+template <> __device__ __forceinline__ void ld2<uint16_t>(const uint16_t* p, float* f) {
+  const uint32_t v = *reinterpret_cast<const uint32_t*>(p);
+  f[0] = __uint_as_float(v << 16); f[1] = __uint_as_float(v & 0xffff0000u);
+}
+template <typename T> __device__ __forceinline__ void st2(T* p, const float* f);
+template <> __device__ __forceinline__ void st2<float>(float* p, const float* f) {
+  *reinterpret_cast<float2*>(p) = make_float2(f[0], f[1]);
+}
+template <> __device__ __forceinline__ void st2<uint16_t>(uint16_t* p, const float* f) {
+  *reinterpret_cast<uint32_t*>(p) = pack_bf16x2(f[0], f[1]);
+}
 
 template <typename T>
 __global__ __launch_bounds__(256) void qknorm_rope_cache_kernel(
@@ -40,45 +58,69 @@ __global__ __launch_bounds__(256) void qknorm_rope_cache_kernel(
   const int rh = rd >> 1;
   const float inv_dk = 1.f / (float)dk;
 
+  // a lane owns the rotation pairs (2i, 2i+1), i = lane + 64 j: one 4-byte (bf16) or 8-byte
+  // (fp32) access per pair when rows and heads start on even elements, values stay in registers
+  // between the sum of squares and the store (dk <= 512)
+  const bool pairvec = ((dk | stride) & 1) == 0;
   for (int head = wave; head < H + G; head += 4) {
     T* hp = row + (size_t)head * dk;                      // q heads, then k heads
     const float* nw = head < H ? qw : kw;
-    float ss = 0.f;
-    for (int e = lane; e < dk; e += 64) {
-      const float x = ldf<T>(hp + e);
-      ss += x * x;
-    }
-    ss = wave_sum(ss);
-    const float r = 1.f / sqrtf(ss * inv_dk + eps);
-    T* dst = nullptr;
+    T* dst = hp;
     if (head >= H) {
       if (slot < 0) continue;
       dst = k_cache + (((size_t)blk * G + (head - H)) * block_size + off) * dk;
     }
-    // the pair partner e ^ 1 lives in the same pass (neighbouring lane): both values are read
-    // before either lane stores
-    for (int e0 = 0; e0 < dk; e0 += 64) {
-      const int e = e0 + lane;
-      float o = 0.f;
-      if (e < dk) {
-        const float x = ldf<T>(hp + e) * r * nw[e];
-        if (e < rd) {
-          const float y = ldf<T>(hp + (e ^ 1)) * r * nw[e ^ 1];
-          const float c = cs[e >> 1], s = cs[rh + (e >> 1)];
-          o = (e & 1) ? x * c + y * s : x * c - y * s;
-        } else {
-          o = x;
-        }
+    float xv[4][2];
+    float ss = 0.f;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int e = 2 * (lane + 64 * j);
+      xv[j][0] = xv[j][1] = 0.f;
+      if (e + 1 < dk && pairvec) {
+        ld2<T>(hp + e, xv[j]);
+      } else if (e < dk) {
+        xv[j][0] = ldf<T>(hp + e);
+        if (e + 1 < dk) xv[j][1] = ldf<T>(hp + e + 1);
       }
-      __builtin_amdgcn_wave_barrier();
-      if (e < dk) stf<T>((dst ? dst : hp) + e, o);
+      ss += xv[j][0] * xv[j][0] + xv[j][1] * xv[j][1];
+    }
+    ss = wave_sum(ss);
+    const float r = 1.f / sqrtf(ss * inv_dk + eps);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int e = 2 * (lane + 64 * j);
+      if (e >= dk) continue;
+      const float x = xv[j][0] * r * nw[e];
+      const float y = e + 1 < dk ? xv[j][1] * r * nw[e + 1] : 0.f;
+      float o[2] = {x, y};
+      if (e + 1 < rd) {
+        const float c = cs[e >> 1], sn = cs[rh + (e >> 1)];
+        o[0] = x * c - y * sn;
+        o[1] = y * c + x * sn;
+      }
+      if (e + 1 < dk && pairvec) {
+        st2<T>(dst + e, o);
+      } else {
+        stf<T>(dst + e, o[0]);
+        if (e + 1 < dk) stf<T>(dst + e + 1, o[1]);
+      }
     }
   }
   if (slot >= 0) {
     const T* vsrc = row + (size_t)(H + G) * dk;
-    for (int i = threadIdx.x; i < G * dv; i += 256) {
-      const int vh = i / dv, d = i - vh * dv;
-      v_cache[(((size_t)blk * G + vh) * block_size + off) * dv + d] = vsrc[i];
+    constexpr int EPV = 16 / sizeof(T);
+    if (dv % EPV == 0 && stride % EPV == 0 && ((H + G) * dk) % EPV == 0 && ((uintptr_t)qkv & 15) == 0) {
+      const int cpv = dv / EPV;
+      for (int i = threadIdx.x; i < G * cpv; i += 256) {
+        const int vh = i / cpv, c = i - vh * cpv;
+        *reinterpret_cast<u32x4*>(v_cache + (((size_t)blk * G + vh) * block_size + off) * dv + c * EPV) =
+            *reinterpret_cast<const u32x4*>(vsrc + (size_t)vh * dv + c * EPV);
+      }
+    } else {
+      for (int i = threadIdx.x; i < G * dv; i += 256) {
+        const int vh = i / dv, d = i - vh * dv;
+        v_cache[(((size_t)blk * G + vh) * block_size + off) * dv + d] = vsrc[i];
+      }
     }
   }
 }
@@ -91,6 +133,7 @@ extern "C" int dgi_qknorm_rope_cache(void* qkv, int is_f32, int T, int stride, c
                                      void* v_cache, int block_size, hipStream_t s) {
   if (T == 0) return 0;
   if (rd < 0 || rd > dk || (rd & 1)) return -2;
+  if (dk > 512) return -3;
   if (is_f32)
     qknorm_rope_cache_kernel<float><<<T, 256, 0, s>>>((float*)qkv, stride, positions, slots, qw, kw, eps, cos_sin,
                                                       rd, H, G, dk, dv, (float*)k_cache, (float*)v_cache, block_size);
