@@ -11,7 +11,7 @@
 //                                                                    norm: one pass over the row)
 //   embed_dyt      res = dyt_a(table[id] * scale)                    (token gather + embedding norm)
 //
-// Elementwise and memory-bound: one workgroup per row, fp32 math with the accurate tanhf (the
+// Elementwise and memory-bound: one workgroup per row, fp32 math (the
 // stream and every norm are kept in 32-bit also when the projections run in bf16).  Norm
 // parameters are fp32; TA is the activation dtype (bf16 bit patterns or float).
 #include "../common.h"
@@ -26,6 +26,14 @@ template <> __device__ __forceinline__ float ldf<uint16_t>(const uint16_t* p) { 
 template <typename T> __device__ __forceinline__ void stf(T* p, float v);
 template <> __device__ __forceinline__ void stf<float>(float* p, float v) { *p = v; }
 template <> __device__ __forceinline__ void stf<uint16_t>(uint16_t* p, float v) { *p = f32_to_bf16(v); }
+
+// tanh(x) = sign(x) (1 - e) / (1 + e), e = exp(-2 |x|) in (0, 1]: the hardware exponential and
+// reciprocal (absolute error below 2e-7, no overflow), a quarter of the instructions of the
+// library tanhf — these kernels evaluate two tanh per element and were ALU-bound on it.
+__device__ __forceinline__ float tanh_fast(float x) {
+  const float e = __expf(-2.f * fabsf(x));
+  return copysignf((1.f - e) * __builtin_amdgcn_rcpf(1.f + e), x);
+}
 
 struct DytParams {
   const float* alpha;   // [1]
@@ -65,11 +73,11 @@ __global__ __launch_bounds__(256) void dyt_kernel(const float* __restrict__ x, D
       float v[4], w[4], b[4], o[4];
       ld4<float>(x + row + c, v); ld4<float>(n.w + c, w); ld4<float>(n.b + c, b);
 #pragma unroll
-      for (int j = 0; j < 4; ++j) o[j] = tanhf(a * v[j]) * w[j] + b[j];
+      for (int j = 0; j < 4; ++j) o[j] = tanh_fast(a * v[j]) * w[j] + b[j];
       st4<TA>(y + row + c, o);
     }
   } else {
-    for (int c = threadIdx.x; c < W; c += 256) stf<TA>(y + row + c, tanhf(a * x[row + c]) * n.w[c] + n.b[c]);
+    for (int c = threadIdx.x; c < W; c += 256) stf<TA>(y + row + c, tanh_fast(a * x[row + c]) * n.w[c] + n.b[c]);
   }
 }
 
@@ -88,23 +96,62 @@ __global__ __launch_bounds__(256) void dyt_add_kernel(const TA* __restrict__ h, 
       ld4<TA>(hr + c, hv); ld4<float>(res + row + c, r);
       ld4<float>(post.w + c, w); ld4<float>(post.b + c, b); ld4<float>(ls + c, l);
 #pragma unroll
-      for (int j = 0; j < 4; ++j) r[j] += (tanhf(a1 * hv[j]) * w[j] + b[j]) * l[j];
+      for (int j = 0; j < 4; ++j) r[j] += (tanh_fast(a1 * hv[j]) * w[j] + b[j]) * l[j];
       st4<float>(res + row + c, r);
       if (y) {
         float o[4];
         ld4<float>(next.w + c, w); ld4<float>(next.b + c, b);
 #pragma unroll
-        for (int j = 0; j < 4; ++j) o[j] = tanhf(a2 * r[j]) * w[j] + b[j];
+        for (int j = 0; j < 4; ++j) o[j] = tanh_fast(a2 * r[j]) * w[j] + b[j];
         st4<TA>(y + row + c, o);
       }
     }
   } else {
     for (int c = threadIdx.x; c < W; c += 256) {
-      const float v = res[row + c] + (tanhf(a1 * ldf<TA>(hr + c)) * post.w[c] + post.b[c]) * ls[c];
+      const float v = res[row + c] + (tanh_fast(a1 * ldf<TA>(hr + c)) * post.w[c] + post.b[c]) * ls[c];
       res[row + c] = v;
-      if (y) stf<TA>(y + row + c, tanhf(a2 * v) * next.w[c] + next.b[c]);
+      if (y) stf<TA>(y + row + c, tanh_fast(a2 * v) * next.w[c] + next.b[c]);
     }
   }
+}
+
+// Tiled form of dyt_add for 16-byte-aligned rows: a thread owns four columns, loads their norm
+// parameters once and walks RPB rows, so the five fp32 parameter vectors (20 bytes per column,
+// more than the 12 bytes per element of data) are read once per RPB rows instead of once per row.
+constexpr int RPB = 8;
+
+template <typename TA>
+__global__ __launch_bounds__(256) void dyt_add_tile_kernel(const TA* __restrict__ h, int h_stride, DytParams post,
+                                                           const float* __restrict__ ls, float* __restrict__ res,
+                                                           DytParams next, TA* __restrict__ y, int T, int W) {
+  const int c = (blockIdx.x * 256 + threadIdx.x) * 4;
+  if (c >= W) return;
+  const int r0 = blockIdx.y * RPB, r1 = min(T, r0 + RPB);
+  const float a1 = post.alpha[0];
+  const float a2 = y ? next.alpha[0] : 0.f;
+  float w1[4], b1[4], l[4], w2[4], b2[4];
+  ld4<float>(post.w + c, w1); ld4<float>(post.b + c, b1); ld4<float>(ls + c, l);
+  if (y) { ld4<float>(next.w + c, w2); ld4<float>(next.b + c, b2); }
+  float hv[RPB][4], rv[RPB][4];
+#pragma unroll
+  for (int i = 0; i < RPB; ++i)
+    if (r0 + i < r1) {
+      ld4<TA>(h + (size_t)(r0 + i) * h_stride + c, hv[i]);
+      ld4<float>(res + (size_t)(r0 + i) * W + c, rv[i]);
+    }
+#pragma unroll
+  for (int i = 0; i < RPB; ++i)
+    if (r0 + i < r1) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) rv[i][j] += (tanh_fast(a1 * hv[i][j]) * w1[j] + b1[j]) * l[j];
+      st4<float>(res + (size_t)(r0 + i) * W + c, rv[i]);
+      if (y) {
+        float o[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) o[j] = tanh_fast(a2 * rv[i][j]) * w2[j] + b2[j];
+        st4<TA>(y + (size_t)(r0 + i) * W + c, o);
+      }
+    }
 }
 
 template <typename TA, bool VEC>
@@ -121,11 +168,11 @@ __global__ __launch_bounds__(256) void embed_dyt_kernel(const long long* __restr
       float v[4], w[4], b[4], o[4];
       ld4<TA>(e + c, v); ld4<float>(n.w + c, w); ld4<float>(n.b + c, b);
 #pragma unroll
-      for (int j = 0; j < 4; ++j) o[j] = tanhf(a * (v[j] * scale)) * w[j] + b[j];
+      for (int j = 0; j < 4; ++j) o[j] = tanh_fast(a * (v[j] * scale)) * w[j] + b[j];
       st4<float>(res + row + c, o);
     }
   } else {
-    for (int c = threadIdx.x; c < W; c += 256) res[row + c] = tanhf(a * (ldf<TA>(e + c) * scale)) * n.w[c] + n.b[c];
+    for (int c = threadIdx.x; c < W; c += 256) res[row + c] = tanh_fast(a * (ldf<TA>(e + c) * scale)) * n.w[c] + n.b[c];
   }
 }
 
@@ -155,6 +202,15 @@ extern "C" int dgi_dyt_add(const void* h, int h_stride, const float* alpha1, con
   const bool vec = W % 4 == 0 && h_stride % 4 == 0 &&
                    ((uintptr_t)h | (uintptr_t)w1 | (uintptr_t)b1 | (uintptr_t)ls | (uintptr_t)res | (uintptr_t)w2 |
                     (uintptr_t)b2 | (uintptr_t)y) % 16 == 0;
+  if (vec && T >= 2 * RPB && (T + RPB - 1) / RPB <= 65535) {
+    const dim3 grid((W / 4 + 255) / 256, (T + RPB - 1) / RPB);
+    if (is_f32)
+      dyt_add_tile_kernel<float><<<grid, 256, 0, s>>>((const float*)h, h_stride, post, ls, res, next, (float*)y, T, W);
+    else
+      dyt_add_tile_kernel<uint16_t><<<grid, 256, 0, s>>>((const uint16_t*)h, h_stride, post, ls, res, next, (uint16_t*)y, T, W);
+    DGI_CHECK_LAUNCH();
+    return 0;
+  }
   if (is_f32) {
     if (vec) dyt_add_kernel<float, true><<<T, 256, 0, s>>>((const float*)h, h_stride, post, ls, res, next, (float*)y, W);
     else dyt_add_kernel<float, false><<<T, 256, 0, s>>>((const float*)h, h_stride, post, ls, res, next, (float*)y, W);

@@ -149,6 +149,228 @@ __global__ __launch_bounds__(64) void masked_attn_rows_kernel(
   }
 }
 
+// ---------------------------------------------------------------------------------------------
+// Grouped kernel: one workgroup per (row, kv head) serves all R = H / G query heads of the group
+// from ONE pass over the keys, with 16-byte cache reads.  Eight waves take 64-key tiles round
+// robin; in a tile lane j scores key j against the R staged queries (its K row is read once),
+// the probabilities go through LDS, and for the values a 16-lane group owns one key at a time
+// (lane c of the group its 16-byte chunk c), so one wave instruction reads four whole V rows.
+// Partial outputs are combined over the four lane groups by shuffles and over the waves in LDS.
+// Needs dk, dv multiples of 8 (bf16) / 4 (fp32), H / G <= 8 and (H / G) * dv <= 1024.
+constexpr int GNW = 8;        // waves per workgroup
+
+template <typename T, int R, int VP>
+__global__ __launch_bounds__(64 * GNW) void masked_attn_group_kernel(
+    const T* __restrict__ q, int q_stride, const T* __restrict__ k_cache, const T* __restrict__ v_cache,
+    const int* __restrict__ block_tables, int bt_stride, const int* __restrict__ cu_seqlens, int n_seqs,
+    const int* __restrict__ positions, int H, int dk, int dv, int bs, float scale, int mask,
+    const T* __restrict__ gate, int gate_stride, T* __restrict__ out, int out_stride) {
+  constexpr int E = 16 / sizeof(T);
+  extern __shared__ __attribute__((aligned(16))) float smem[];
+  const int row = blockIdx.x, kvh = blockIdx.y, G = gridDim.y;
+  const int r = H / G;
+  const int tid = threadIdx.x, w = tid >> 6, lane = tid & 63;
+  const int lg = lane >> 4, lc = lane & 15;
+  float* qs = smem;                                  // [R][dk]
+  float* ps = qs + R * dk;                           // [GNW][R][64]
+  int* vs = reinterpret_cast<int*>(ps + GNW * R * 64);   // [GNW][64] cache slot of each key of the wave's tile
+  float* cm = reinterpret_cast<float*>(vs + GNW * 64);   // [GNW][R] running max, then [GNW][R] sums
+  float* co = cm + 2 * GNW * R;                      // [GNW][R][dv] partial outputs
+
+  int seq = row;
+  if (cu_seqlens) {
+    int lo = 0, hi = n_seqs - 1;
+    while (lo < hi) {
+      const int mid = (lo + hi + 1) >> 1;
+      if (cu_seqlens[mid] <= row) lo = mid; else hi = mid - 1;
+    }
+    seq = lo;
+  }
+  const int* bt = block_tables + (size_t)seq * bt_stride;
+  const int pos = positions[row];
+  const int first = mask > 0 ? (pos / mask) * mask : 0;
+
+  const T* qp = q + (size_t)row * q_stride + (size_t)kvh * r * dk;
+  for (int e = tid; e < r * dk; e += 64 * GNW) qs[e] = ldf<T>(qp + e);
+  __syncthreads();
+
+  float m[R], l[R], o[R][VP][E];
+#pragma unroll
+  for (int i = 0; i < R; ++i) {
+    m[i] = -__builtin_inff();
+    l[i] = 0.f;
+#pragma unroll
+    for (int p = 0; p < VP; ++p)
+#pragma unroll
+      for (int j = 0; j < E; ++j) o[i][p][j] = 0.f;
+  }
+  float* psw = ps + w * R * 64;
+  int* vsw = vs + w * 64;
+  const int ntiles = (pos - first) / 64 + 1;
+  for (int tile = w; tile < ntiles; tile += GNW) {
+    const int k0 = first + tile * 64;
+    const int key = k0 + lane;
+    const bool ok = key <= pos;
+    float sc[R];
+#pragma unroll
+    for (int i = 0; i < R; ++i) sc[i] = 0.f;
+    int slot = 0;
+    if (ok) {
+      slot = (bt[key / bs] * G + kvh) * bs + (key % bs);
+      const T* kp = k_cache + (size_t)slot * dk;
+      for (int e = 0; e < dk; e += E) {
+        float kf[E];
+        const u32x4 kv = *reinterpret_cast<const u32x4*>(kp + e);
+        if constexpr (sizeof(T) == 2) {
+          unpack8(kv, kf);
+        } else {
+#pragma unroll
+          for (int j = 0; j < 4; ++j) kf[j] = __uint_as_float(kv[j]);
+        }
+#pragma unroll
+        for (int i = 0; i < R; ++i) {
+          if (i < r) {
+            const float* qi = qs + i * dk + e;
+#pragma unroll
+            for (int j = 0; j < E; ++j) sc[i] += qi[j] * kf[j];
+          }
+        }
+      }
+    }
+    // this wave's previous tile is fully consumed (its LDS reads were issued, in order, before)
+#pragma unroll
+    for (int i = 0; i < R; ++i) {
+      if (i < r) {
+        const float s = ok ? sc[i] * scale : -__builtin_inff();
+        const float m_new = fmaxf(m[i], wave_max(s));       // key k0 (lane 0) is visible: finite
+        const float p = ok ? expf(s - m_new) : 0.f;
+        const float corr = expf(m[i] - m_new);
+        l[i] = l[i] * corr + wave_sum(p);
+        m[i] = m_new;
+#pragma unroll
+        for (int vp = 0; vp < VP; ++vp)
+#pragma unroll
+          for (int j = 0; j < E; ++j) o[i][vp][j] *= corr;
+        psw[i * 64 + lane] = p;
+      }
+    }
+    vsw[lane] = slot;
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    const int n = min(64, pos - k0 + 1);
+    for (int kk = lg; kk < n; kk += 4) {
+      const T* vp_ = v_cache + (size_t)vsw[kk] * dv;
+      float pk[R];
+#pragma unroll
+      for (int i = 0; i < R; ++i) pk[i] = i < r ? psw[i * 64 + kk] : 0.f;
+#pragma unroll
+      for (int vp = 0; vp < VP; ++vp) {
+        const int c = (lc + 16 * vp) * E;
+        if (c < dv) {
+          float vf[E];
+          const u32x4 vv = *reinterpret_cast<const u32x4*>(vp_ + c);
+          if constexpr (sizeof(T) == 2) {
+            unpack8(vv, vf);
+          } else {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) vf[j] = __uint_as_float(vv[j]);
+          }
+#pragma unroll
+          for (int i = 0; i < R; ++i)
+#pragma unroll
+            for (int j = 0; j < E; ++j) o[i][vp][j] += pk[i] * vf[j];
+        }
+      }
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+  }
+  // lane groups -> lane group 0, then waves -> LDS
+#pragma unroll
+  for (int i = 0; i < R; ++i)
+#pragma unroll
+    for (int vp = 0; vp < VP; ++vp)
+#pragma unroll
+      for (int j = 0; j < E; ++j) {
+        float v = o[i][vp][j];
+        v += __shfl_xor(v, 16, 64);
+        v += __shfl_xor(v, 32, 64);
+        o[i][vp][j] = v;
+      }
+  if (lane == 0) {
+#pragma unroll
+    for (int i = 0; i < R; ++i) {
+      cm[w * R + i] = m[i];
+      cm[GNW * R + w * R + i] = l[i];
+    }
+  }
+  if (lg == 0) {
+#pragma unroll
+    for (int i = 0; i < R; ++i)
+      if (i < r)
+#pragma unroll
+        for (int vp = 0; vp < VP; ++vp) {
+          const int c = (lc + 16 * vp) * E;
+          if (c < dv)
+#pragma unroll
+            for (int j = 0; j < E; ++j) co[((size_t)w * R + i) * dv + c + j] = o[i][vp][j];
+        }
+  }
+  __syncthreads();
+  for (int idx = tid; idx < r * dv; idx += 64 * GNW) {
+    const int i = idx / dv, d = idx - i * dv;
+    float M = -__builtin_inff();
+#pragma unroll
+    for (int ww = 0; ww < GNW; ++ww) M = fmaxf(M, cm[ww * R + i]);
+    float L = 0.f, O = 0.f;
+#pragma unroll
+    for (int ww = 0; ww < GNW; ++ww) {
+      const float f = expf(cm[ww * R + i] - M);          // waves without a tile: exp(-inf) = 0
+      L += cm[GNW * R + ww * R + i] * f;
+      O += co[((size_t)ww * R + i) * dv + d] * f;
+    }
+    float v = O / L;
+    const int head = kvh * r + i;
+    if (gate) v *= 1.f / (1.f + expf(-ldf<T>(gate + (size_t)row * gate_stride + (size_t)head * dv + d)));
+    stf<T>(out + (size_t)row * out_stride + (size_t)head * dv + d, v);
+  }
+}
+
+template <typename T, int R, int VP>
+int launch_group(const void* q, int q_stride, const void* k_cache, const void* v_cache, const int* block_tables,
+                 int bt_stride, const int* cu_seqlens, int n_seqs, const int* positions, int rows, int H, int G, int dk,
+                 int dv, int bs, float scale, int mask, const void* gate, int gate_stride, void* out, int out_stride,
+                 hipStream_t s) {
+  const size_t lds = (size_t)(R * dk + GNW * R * 64 + GNW * 64 + 2 * GNW * R + GNW * R * dv) * 4;
+  if (lds > 64 * 1024) return -1;
+  masked_attn_group_kernel<T, R, VP><<<dim3(rows, G), 64 * GNW, lds, s>>>(
+      (const T*)q, q_stride, (const T*)k_cache, (const T*)v_cache, block_tables, bt_stride, cu_seqlens, n_seqs,
+      positions, H, dk, dv, bs, scale, mask, (const T*)gate, gate_stride, (T*)out, out_stride);
+  return 0;
+}
+
+template <typename T>
+int dispatch_group(int r, int vpn, const void* q, int q_stride, const void* k_cache, const void* v_cache,
+                   const int* block_tables, int bt_stride, const int* cu_seqlens, int n_seqs, const int* positions,
+                   int rows, int H, int G, int dk, int dv, int bs, float scale, int mask, const void* gate,
+                   int gate_stride, void* out, int out_stride, hipStream_t s) {
+#define DGI_GRP(RV, VPV)                                                                                       \
+  return launch_group<T, RV, VPV>(q, q_stride, k_cache, v_cache, block_tables, bt_stride, cu_seqlens, n_seqs, \
+                                  positions, rows, H, G, dk, dv, bs, scale, mask, gate, gate_stride, out, out_stride, s)
+  if (vpn == 1) {
+    if (r == 1) DGI_GRP(1, 1);
+    if (r == 2) DGI_GRP(2, 1);
+    if (r <= 4) DGI_GRP(4, 1);
+    DGI_GRP(8, 1);
+  }
+  if (r == 1) DGI_GRP(1, 2);
+  if (r == 2) DGI_GRP(2, 2);
+  if (r <= 4) DGI_GRP(4, 2);
+  DGI_GRP(8, 2);
+#undef DGI_GRP
+}
+
 }  // namespace
 
 // q / gate / out: row-major with their own row strides (elements); cu_seqlens (n_seqs + 1 row
@@ -162,6 +384,24 @@ extern "C" int dgi_masked_attn_rows(const void* q, int q_stride, const void* k_c
   if (G <= 0 || H % G) return -2;
   if (dk > MAXDK || dv > 64 * MAXC || dk <= 0 || dv <= 0) return -3;
   if (H > 65535 || mask < 0) return -4;
+  {
+    // grouped kernel where the geometry allows (see masked_attn_group_kernel)
+    const int E = is_f32 ? 4 : 8, r = H / G;
+    const int vpn = (dv + 16 * E - 1) / (16 * E);
+    const bool aligned = ((uintptr_t)k_cache | (uintptr_t)v_cache) % 16 == 0;
+    if (dk % E == 0 && dv % E == 0 && r <= 8 && vpn <= 2 && r * dv <= 1024 && aligned && G <= 65535) {
+      const int rc = is_f32 ? dispatch_group<float>(r, vpn, q, q_stride, k_cache, v_cache, block_tables, bt_stride, cu_seqlens,
+                                                    n_seqs, positions, rows, H, G, dk, dv, block_size, scale, mask, gate,
+                                                    gate_stride, out, out_stride, s)
+                            : dispatch_group<uint16_t>(r, vpn, q, q_stride, k_cache, v_cache, block_tables, bt_stride,
+                                                       cu_seqlens, n_seqs, positions, rows, H, G, dk, dv, block_size, scale,
+                                                       mask, gate, gate_stride, out, out_stride, s);
+      if (rc == 0) {
+        DGI_CHECK_LAUNCH();
+        return 0;
+      }
+    }
+  }
   const dim3 grid(rows, H);
   if (is_f32)
     masked_attn_rows_kernel<float><<<grid, 64, 0, s>>>(

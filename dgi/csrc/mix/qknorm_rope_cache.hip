@@ -125,6 +125,107 @@ __global__ __launch_bounds__(256) void qknorm_rope_cache_kernel(
   }
 }
 
+// Sixteen lanes per head, 16-byte chunks (dk a multiple of 8 bf16 / 4 fp32): a workgroup
+// normalises sixteen heads of one token at once (grid.y walks the heads), each lane keeps up to
+// MAXCH chunks in registers between the sum of squares (four shuffles inside the 16-lane
+// group) and the store; norm weights and cos / sin come in as 16-byte loads.
+template <typename T, int MAXCH>
+__global__ __launch_bounds__(256) void qknorm_rope_cache_vec_kernel(
+    T* __restrict__ qkv, int stride, const int* __restrict__ positions, const int* __restrict__ slots,
+    const float* __restrict__ qw, const float* __restrict__ kw, float eps, const float* __restrict__ cos_sin,
+    int rd, int H, int G, int dk, int dv, T* __restrict__ k_cache, T* __restrict__ v_cache, int block_size) {
+  constexpr int E = 16 / sizeof(T);
+  const int t = blockIdx.x;
+  const int grp = threadIdx.x >> 4, l = threadIdx.x & 15;
+  T* row = qkv + (size_t)t * stride;
+  const int slot = slots ? slots[t] : -1;
+  const int blk = slot >= 0 ? slot / block_size : 0;
+  const int off = slot >= 0 ? slot - blk * block_size : 0;
+  const float* cs = rd > 0 ? cos_sin + (size_t)positions[t] * rd : nullptr;
+  const int rh = rd >> 1;
+  const float inv_dk = 1.f / (float)dk;
+  const int nch = dk / E;
+
+  const int head = blockIdx.y * 16 + grp;               // grid.y covers the heads sixteen at a time
+  if (head < H + G && !(head >= H && slot < 0)) {
+    T* hp = row + (size_t)head * dk;
+    const float* nw = head < H ? qw : kw;
+    T* dst = hp;
+    if (head >= H) dst = k_cache + (((size_t)blk * G + (head - H)) * block_size + off) * dk;
+    const bool csvec = (rd & 7) == 0 && E == 8;         // four cos + four sin of a chunk as two float4
+    float x[MAXCH][E];
+    float ss = 0.f;
+#pragma unroll
+    for (int j = 0; j < MAXCH; ++j) {
+      const int c = l + 16 * j;
+      if (c < nch) {
+        const u32x4 v = *reinterpret_cast<const u32x4*>(hp + c * E);
+        if constexpr (sizeof(T) == 2) {
+          unpack8(v, x[j]);
+        } else {
+#pragma unroll
+          for (int i = 0; i < 4; ++i) x[j][i] = __uint_as_float(v[i]);
+        }
+#pragma unroll
+        for (int i = 0; i < E; ++i) ss += x[j][i] * x[j][i];
+      }
+    }
+#pragma unroll
+    for (int o = 8; o > 0; o >>= 1) ss += __shfl_xor(ss, o, 64);
+    const float r = 1.f / sqrtf(ss * inv_dk + eps);
+#pragma unroll
+    for (int j = 0; j < MAXCH; ++j) {
+      const int c = l + 16 * j;
+      if (c >= nch) continue;
+      const int e0 = c * E;
+      float o[E], wv[E], cv[E / 2], sv[E / 2];
+#pragma unroll
+      for (int i = 0; i < E; i += 4) *reinterpret_cast<float4*>(wv + i) = *reinterpret_cast<const float4*>(nw + e0 + i);
+      if (csvec && e0 + E <= rd) {
+        *reinterpret_cast<float4*>(cv) = *reinterpret_cast<const float4*>(cs + (e0 >> 1));
+        *reinterpret_cast<float4*>(sv) = *reinterpret_cast<const float4*>(cs + rh + (e0 >> 1));
+      } else {
+#pragma unroll
+        for (int i = 0; i < E / 2; ++i) {
+          const bool rot = e0 + 2 * i + 1 < rd;
+          cv[i] = rot ? cs[(e0 >> 1) + i] : 1.f;
+          sv[i] = rot ? cs[rh + (e0 >> 1) + i] : 0.f;
+        }
+      }
+#pragma unroll
+      for (int i = 0; i < E; i += 2) {
+        const float a = x[j][i] * r * wv[i], b = x[j][i + 1] * r * wv[i + 1];
+        o[i] = a * cv[i >> 1] - b * sv[i >> 1];
+        o[i + 1] = b * cv[i >> 1] + a * sv[i >> 1];
+      }
+      u32x4 w;
+      if constexpr (sizeof(T) == 2) {
+        w = pack8(o);
+      } else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) w[i] = __float_as_uint(o[i]);
+      }
+      *reinterpret_cast<u32x4*>(dst + e0) = w;
+    }
+  }
+  if (slot >= 0 && blockIdx.y == 0) {
+    const T* vsrc = row + (size_t)(H + G) * dk;
+    if (dv % E == 0) {
+      const int cpv = dv / E;
+      for (int i = threadIdx.x; i < G * cpv; i += 256) {
+        const int vh = i / cpv, c = i - vh * cpv;
+        *reinterpret_cast<u32x4*>(v_cache + (((size_t)blk * G + vh) * block_size + off) * dv + c * E) =
+            *reinterpret_cast<const u32x4*>(vsrc + (size_t)vh * dv + c * E);
+      }
+    } else {
+      for (int i = threadIdx.x; i < G * dv; i += 256) {
+        const int vh = i / dv, d = i - vh * dv;
+        v_cache[(((size_t)blk * G + vh) * block_size + off) * dv + d] = vsrc[i];
+      }
+    }
+  }
+}
+
 }  // namespace
 
 extern "C" int dgi_qknorm_rope_cache(void* qkv, int is_f32, int T, int stride, const int* positions,
@@ -134,6 +235,20 @@ extern "C" int dgi_qknorm_rope_cache(void* qkv, int is_f32, int T, int stride, c
   if (T == 0) return 0;
   if (rd < 0 || rd > dk || (rd & 1)) return -2;
   if (dk > 512) return -3;
+  const int E = is_f32 ? 4 : 8;
+  if (dk % E == 0 && stride % E == 0 && dk <= 64 * E && ((uintptr_t)qkv | (uintptr_t)k_cache | (uintptr_t)v_cache) % 16 == 0) {
+    if ((H + G + 15) / 16 > 65535) return -4;
+    const dim3 vgrid(T, (H + G + 15) / 16);
+    if (is_f32)
+      qknorm_rope_cache_vec_kernel<float, 4><<<vgrid, 256, 0, s>>>((float*)qkv, stride, positions, slots, qw, kw, eps, cos_sin,
+                                                               rd, H, G, dk, dv, (float*)k_cache, (float*)v_cache, block_size);
+    else
+      qknorm_rope_cache_vec_kernel<uint16_t, 4><<<vgrid, 256, 0, s>>>((uint16_t*)qkv, stride, positions, slots, qw, kw, eps,
+                                                                  cos_sin, rd, H, G, dk, dv, (uint16_t*)k_cache,
+                                                                  (uint16_t*)v_cache, block_size);
+    DGI_CHECK_LAUNCH();
+    return 0;
+  }
   if (is_f32)
     qknorm_rope_cache_kernel<float><<<T, 256, 0, s>>>((float*)qkv, stride, positions, slots, qw, kw, eps, cos_sin,
                                                       rd, H, G, dk, dv, (float*)k_cache, (float*)v_cache, block_size);

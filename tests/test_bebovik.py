@@ -76,9 +76,10 @@ def close(a, b, tol):
 # ----------------------------------------------------------------------------------- mechanisms
 @pytest.mark.parametrize("device", DEVICES)
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-def test_dyt_norms(device, dtype):
+@pytest.mark.parametrize("shape", [(5, 70), (37, 72), (16, 1032)])
+def test_dyt_norms(device, dtype, shape):
     g = torch.Generator().manual_seed(1)
-    T, W = 5, 70
+    T, W = shape             # scalar path, 16-byte path, and the row-tiled path with a ragged last tile
     mk = lambda: DytNorm(torch.rand(1, generator=g).add(0.3).to(device), torch.randn(W, generator=g).to(device),   # noqa: E731
                          torch.randn(W, generator=g).to(device))
     n1, n2 = mk(), mk()
