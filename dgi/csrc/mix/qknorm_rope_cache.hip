@@ -130,7 +130,7 @@ __global__ __launch_bounds__(256) void qknorm_rope_cache_kernel(
 // MAXCH chunks in registers between the sum of squares (four shuffles inside the 16-lane
 // group) and the store; norm weights and cos / sin come in as 16-byte loads.
 template <typename T, int MAXCH>
-__global__ __launch_bounds__(256) void qknorm_rope_cache_vec_kernel(
+__global__ __launch_bounds__(1024) void qknorm_rope_cache_vec_kernel(
     T* __restrict__ qkv, int stride, const int* __restrict__ positions, const int* __restrict__ slots,
     const float* __restrict__ qw, const float* __restrict__ kw, float eps, const float* __restrict__ cos_sin,
     int rd, int H, int G, int dk, int dv, T* __restrict__ k_cache, T* __restrict__ v_cache, int block_size) {
@@ -146,7 +146,7 @@ __global__ __launch_bounds__(256) void qknorm_rope_cache_vec_kernel(
   const float inv_dk = 1.f / (float)dk;
   const int nch = dk / E;
 
-  const int head = blockIdx.y * 16 + grp;               // grid.y covers the heads sixteen at a time
+  const int head = blockIdx.y * (blockDim.x >> 4) + grp;  // blockDim / 16 heads per workgroup, grid.y for the rest
   if (head < H + G && !(head >= H && slot < 0)) {
     T* hp = row + (size_t)head * dk;
     const float* nw = head < H ? qw : kw;
@@ -212,13 +212,13 @@ __global__ __launch_bounds__(256) void qknorm_rope_cache_vec_kernel(
     const T* vsrc = row + (size_t)(H + G) * dk;
     if (dv % E == 0) {
       const int cpv = dv / E;
-      for (int i = threadIdx.x; i < G * cpv; i += 256) {
+      for (int i = threadIdx.x; i < G * cpv; i += blockDim.x) {
         const int vh = i / cpv, c = i - vh * cpv;
         *reinterpret_cast<u32x4*>(v_cache + (((size_t)blk * G + vh) * block_size + off) * dv + c * E) =
             *reinterpret_cast<const u32x4*>(vsrc + (size_t)vh * dv + c * E);
       }
     } else {
-      for (int i = threadIdx.x; i < G * dv; i += 256) {
+      for (int i = threadIdx.x; i < G * dv; i += blockDim.x) {
         const int vh = i / dv, d = i - vh * dv;
         v_cache[(((size_t)blk * G + vh) * block_size + off) * dv + d] = vsrc[i];
       }
@@ -237,13 +237,16 @@ extern "C" int dgi_qknorm_rope_cache(void* qkv, int is_f32, int T, int stride, c
   if (dk > 512) return -3;
   const int E = is_f32 ? 4 : 8;
   if (dk % E == 0 && stride % E == 0 && dk <= 64 * E && ((uintptr_t)qkv | (uintptr_t)k_cache | (uintptr_t)v_cache) % 16 == 0) {
-    if ((H + G + 15) / 16 > 65535) return -4;
-    const dim3 vgrid(T, (H + G + 15) / 16);
+    // one workgroup per token when its heads fit 1024 threads (16 lanes each), else grid.y more
+    const int hpb = (H + G) < 64 ? (H + G) : 64;
+    const int vthreads = (hpb * 16 + 63) / 64 * 64;
+    if ((H + G + hpb - 1) / hpb > 65535) return -4;
+    const dim3 vgrid(T, (H + G + hpb - 1) / hpb);
     if (is_f32)
-      qknorm_rope_cache_vec_kernel<float, 4><<<vgrid, 256, 0, s>>>((float*)qkv, stride, positions, slots, qw, kw, eps, cos_sin,
+      qknorm_rope_cache_vec_kernel<float, 4><<<vgrid, vthreads, 0, s>>>((float*)qkv, stride, positions, slots, qw, kw, eps, cos_sin,
                                                                rd, H, G, dk, dv, (float*)k_cache, (float*)v_cache, block_size);
     else
-      qknorm_rope_cache_vec_kernel<uint16_t, 4><<<vgrid, 256, 0, s>>>((uint16_t*)qkv, stride, positions, slots, qw, kw, eps,
+      qknorm_rope_cache_vec_kernel<uint16_t, 4><<<vgrid, vthreads, 0, s>>>((uint16_t*)qkv, stride, positions, slots, qw, kw, eps,
                                                                   cos_sin, rd, H, G, dk, dv, (uint16_t*)k_cache,
                                                                   (uint16_t*)v_cache, block_size);
     DGI_CHECK_LAUNCH();

@@ -97,7 +97,8 @@ def dyt_add(res: torch.Tensor, h: torch.Tensor, post: DytNorm, ls: torch.Tensor,
 
 
 def embed_dyt_ref(ids: torch.Tensor, table: torch.Tensor, scale: float, n: DytNorm) -> torch.Tensor:
-    return dyt_ref(table[ids.long()].float() * scale, n, torch.float32)
+    ids = ids.long().clamp(0, table.shape[0] - 1)          # the kernel clamps too: no read outside the table
+    return dyt_ref(table[ids].float() * scale, n, torch.float32)
 
 
 def embed_dyt(ids: torch.Tensor, table: torch.Tensor, scale: float, n: DytNorm) -> torch.Tensor:

@@ -51,6 +51,45 @@ def xcd_split(n_cus: int, side_per_xcd: int, xcds: int = 8) -> tuple:
     return [c for c in range(n_cus) if c not in ss], side
 
 
+_CU_MASK_OK: dict = {}
+
+
+def cu_mask_supported(device_index: int = 0) -> bool:
+    """Whether a serving process of this user can create the pair of CU-masked streams the
+    two-batch overlap needs.  Probed once, in a child process that does what the caller is about
+    to do (PyTorch initialised on the device, two masked streams, one kernel): where the driver
+    refuses a masked queue, the refused creation leaves the process that tried it unable to
+    allocate device memory afterwards, so the serving process never tries it first itself."""
+    hit = _CU_MASK_OK.get(device_index)
+    if hit is None:
+        import os
+        import subprocess
+        import sys
+        root = os.path.dirname(os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
+        i = int(device_index)
+        code = ("import sys, torch\n"
+                f"sys.path.insert(0, {root!r})\n"
+                f"torch.cuda.set_device({i})\n"
+                "x = torch.zeros(8, device='cuda')\n"
+                "from dgi.utils import streams\n"
+                f"streams._CU_MASK_OK[{i}] = True\n"
+                "n = torch.cuda.get_device_properties(0).multi_processor_count\n"
+                "main, side = streams.xcd_split(n, 4)\n"
+                f"a = streams.cu_masked_stream('probe_a', 'cuda:{i}', main)\n"
+                f"b = streams.cu_masked_stream('probe_b', 'cuda:{i}', side)\n"
+                "with torch.cuda.stream(b):\n"
+                "    y = torch.ones(1024, device='cuda').sum()\n"
+                "torch.cuda.synchronize()\n"
+                "sys.exit(0 if float(y) == 1024.0 else 3)\n")
+        try:
+            hit = subprocess.run([sys.executable, "-c", code], timeout=300, stdin=subprocess.DEVNULL,
+                                 stdout=subprocess.DEVNULL, stderr=subprocess.DEVNULL).returncode == 0
+        except Exception:
+            hit = False
+        _CU_MASK_OK[device_index] = hit
+    return hit
+
+
 def cu_masked_stream(name: str, device, cus: list) -> "torch.cuda.ExternalStream":
     """A stream whose kernels run only on CUs ``cus`` (``hipExtStreamCreateWithCUMask``).
 
@@ -64,6 +103,8 @@ def cu_masked_stream(name: str, device, cus: list) -> "torch.cuda.ExternalStream
     hit = _STREAMS.get(key)
     if hit is not None:
         return hit[0]
+    if not cu_mask_supported(idx):
+        raise RuntimeError(f"hipExtStreamCreateWithCUMask({name}): CU-masked streams are refused on this machine")
     n = torch.cuda.get_device_properties(idx).multi_processor_count
     words = [0] * ((n + 31) // 32)
     for c in cus:

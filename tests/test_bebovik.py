@@ -508,3 +508,36 @@ def test_trace_runner_cli(tmp_path, device):
     close(rd(0), w1[[0, 8]], 3e-4)
     close(rd(1), w2[[1]], 3e-4)
     close(rd(2), torch.cat([w2[[6]], w1[[9]]]), 3e-4)
+
+
+def test_worker_engine_serves_a_checkpoint_dir(tmp_path):
+    """The worker's native engine picks the model class from config.json and generates through
+    the same LLMEngine (chat template, tokenizer fallback, prefix caching on by default)."""
+    sys.path.insert(0, os.path.join(ROOT, "worker"))
+    from engines.llm_native import NativeLLMEngine
+    cfg = small_cfg()
+    d = str(tmp_path / "ckpt")
+    _save_design(engine(cfg, "cpu", torch.bfloat16).model, cfg, d)
+    e = NativeLLMEngine({"model_id": d, "device": "cpu", "max_model_len": 128, "max_num_batched_tokens": 128,
+                         "num_blocks": 64, "max_num_seqs": 4})
+    e.load_model()
+    assert type(e.engine.model).__name__ == "BebovikModel"
+    out = e.batch_inference([{"messages": [{"role": "user", "content": "hi"}], "max_tokens": 5, "temperature": 0.0}])
+    assert out[0]["usage"]["completion_tokens"] == 5
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_prefix_cache_hit_generates_the_same_tokens(device):
+    cfg = small_cfg()
+    eng = LLMEngine(EngineConfig(model="bebovik-test", device=device, dtype=torch.float32, block_size=4, num_blocks=64,
+                                 max_num_seqs=4, max_model_len=128, max_num_batched_tokens=128, enable_prefix_caching=True,
+                                 use_graphs=False, seed=3), model_cfg=cfg)
+    p = toks(30, 60)
+    sp = SamplingParams(max_tokens=6, temperature=0.0, ignore_eos=True)
+    a = eng.generate([p], sp)[0]
+    b = eng.generate([p + [5, 6]], sp)[0]
+    c = eng.generate([p], sp)[0]
+    assert c.num_cached >= 24 and b.num_cached >= 24 and a.num_cached == 0
+    assert c.output == a.output
+    fresh = engine(cfg, device)
+    assert fresh.generate([p + [5, 6]], sp)[0].output == b.output

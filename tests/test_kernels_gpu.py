@@ -814,7 +814,12 @@ def test_two_batch_overlap_decode_step_matches_one_batch(rows, monkeypatch):
     monkeypatch.setattr(llama, "TBO", True)
     assert eng.model._tbo_ok(torch.empty(rows, 8, device="cuda", dtype=torch.bfloat16), meta, None) == \
         llama.tbo_split(rows)
-    got = eng.model.forward(meta, input_ids=ids).float()
+    try:
+        got = eng.model.forward(meta, input_ids=ids).float()
+    except RuntimeError as e:
+        if "hipExtStreamCreateWithCUMask" in str(e):     # the box refuses CU-masked queues to this user
+            pytest.skip(f"CU-masked streams unavailable here: {e}")
+        raise
     torch.cuda.synchronize()
     scale = float(ref.abs().max())
     assert float((got - ref).abs().max()) <= 0.02 * scale

@@ -160,8 +160,9 @@ def cmd_install(a) -> int:
     print("all required packages present")
     try:
         sys.path.insert(0, os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
-        from dgi.build import build
-        build()
+        from dgi.build import GROUPS, build
+        for g in GROUPS:
+            build(group=g)
         print("dgi HIP kernels built for gfx950")
     except Exception as e:
         print("dgi kernels not built:", e)
