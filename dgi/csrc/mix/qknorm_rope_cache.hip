@@ -13,6 +13,7 @@
 // Cache layout per layer: k [num_blocks, G, block_size, dk], v [num_blocks, G, block_size, dv].
 // One workgroup per token; a wave owns one head at a time (sum of squares by wave reduction),
 // a lane its rotation pairs; v rows are copied in 16-byte chunks where the sizes allow.
+#include <cstdlib>
 #include "../common.h"
 
 using namespace dgi;
@@ -237,8 +238,11 @@ extern "C" int dgi_qknorm_rope_cache(void* qkv, int is_f32, int T, int stride, c
   if (dk > 512) return -3;
   const int E = is_f32 ? 4 : 8;
   if (dk % E == 0 && stride % E == 0 && dk <= 64 * E && ((uintptr_t)qkv | (uintptr_t)k_cache | (uintptr_t)v_cache) % 16 == 0) {
-    // one workgroup per token when its heads fit 1024 threads (16 lanes each), else grid.y more
-    const int hpb = (H + G) < 64 ? (H + G) : 64;
+    // heads per workgroup (16 lanes each): 4 to 16 measured alike on 8B-class rows (36-39 us for
+    // 8192 tokens), 32 and more slower (bigger workgroups hide less latency); DGI_QKNORM_HPB for sweeps
+    static const int hpb_env = [] { const char* e = getenv("DGI_QKNORM_HPB"); return e ? atoi(e) : 0; }();
+    int hpb = hpb_env > 0 ? (hpb_env > 64 ? 64 : hpb_env) : 8;
+    if (hpb > H + G) hpb = H + G;
     const int vthreads = (hpb * 16 + 63) / 64 * 64;
     if ((H + G + hpb - 1) / hpb > 65535) return -4;
     const dim3 vgrid(T, (H + G + hpb - 1) / hpb);

@@ -212,7 +212,7 @@ class BebovikModel:
     @staticmethod
     def _mfma_prefill_ok(m, q: torch.Tensor, kc: torch.Tensor) -> bool:
         return (q.is_cuda and q.dtype == torch.bfloat16 and m.dim == m.vdim and m.dim in (64, 128)
-                and ops.masked_prefill_available())
+                and mix.masked_prefill_available())
 
     def attention(self, li: int, qkvg: torch.Tensor, meta: AttnMeta) -> torch.Tensor:
         """Gated attention output [T, H * dv] of the fused projection rows [q | k | v | g]."""
@@ -232,7 +232,7 @@ class BebovikModel:
                                  m.kv_heads, m.scale, mask, None if gate is None else gate[:nd], out=out[:nd])
         if meta.num_prefill_tokens > 0:
             if self._mfma_prefill_ok(m, qkvg, kc):
-                ops.paged_prefill_masked(qkvg[nd:], kc, vc, meta.pre_block_tables, meta.pre_cu_seqlens,
+                mix.paged_prefill_masked(qkvg[nd:], kc, vc, meta.pre_block_tables, meta.pre_cu_seqlens,
                                          meta.pre_context_lens, m.heads, m.kv_heads, m.scale, mask,
                                          None if gate is None else gate[nd:], tiles=meta.pre_tiles, out=out[nd:])
             else:

@@ -370,43 +370,6 @@ def paged_prefill(q, k_cache, v_cache, block_tables, cu_seqlens_q, context_lens,
     return r
 
 
-MASKED_PREFILL = os.environ.get("DGI_MASKED_PREFILL", "1") == "1"   # 0: prompt rows on the row-wise kernel (A/B)
-
-
-def masked_prefill_available() -> bool:
-    """Whether prompt portions may take the MFMA kernel with a block mask and gate epilogue."""
-    return MASKED_PREFILL and PREFILL_TILE == 128
-
-
-def paged_prefill_masked(q, k_cache, v_cache, block_tables, cu_seqlens_q, context_lens, nh, nkv, scale,
-                         mask: int = 0, gate=None, tiles=None, out=None) -> torch.Tensor:
-    """``paged_prefill`` with a block mask — a query at position p sees keys
-    [floor(p / mask) * mask, p] (``mask`` 0: all keys up to p) — and an optional sigmoid output
-    gate (out *= sigmoid(gate)).  bf16, key size == value size in {64, 128} on the GPU
-    (dgi/csrc/mix/masked_prefill.hip); the row-wise reference elsewhere."""
-    from dgi.ops import mix
-    if _native(q):
-        mix.load_native(required=True)
-        hd = k_cache.shape[-1]
-        if out is None:
-            out = torch.empty(q.shape[0], nh * hd, dtype=q.dtype, device=q.device)
-        if tiles is None:
-            tl = prefill_tiles(cu_seqlens_q.tolist(), context_lens=context_lens.tolist(), tile=128)
-            tiles = torch.tensor(tl if tl else [[0, 0]], dtype=torch.int32, device=q.device)[: len(tl)]
-        _call("paged_prefill_masked", out, q, k_cache, v_cache, block_tables, cu_seqlens_q, context_lens, tiles,
-              nh, nkv, float(scale), int(mask), gate)
-        return out
-    cu = cu_seqlens_q.tolist()
-    pos = torch.cat([torch.arange(int(context_lens[b]) - (cu[b + 1] - cu[b]), int(context_lens[b]), dtype=torch.int32)
-                     for b in range(len(cu) - 1)]) if len(cu) > 1 else torch.zeros(0, dtype=torch.int32)
-    r = mix.masked_attn_rows_ref(q, k_cache, v_cache, block_tables, cu_seqlens_q, pos.to(q.device), nh, nkv, scale,
-                                 mask, gate)
-    if out is not None:
-        out.copy_(r)
-        return out
-    return r
-
-
 # ----------------------------------------------------------------------------
 # MLP activation
 # ----------------------------------------------------------------------------
@@ -449,8 +412,8 @@ def linear(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None
     M, K = x.shape
     N = w.shape[0]
     if (x.is_cuda and _use_skinny(M, N, K) and x.dtype == torch.bfloat16
-            and w.dtype == torch.bfloat16 and x.stride(1) == 1 and x.stride(0) % 8 == 0 and w.is_contiguous()):
-        load_native(required=True)
+            and w.dtype == torch.bfloat16 and x.stride(1) == 1 and x.stride(0) % 8 == 0 and w.is_contiguous()
+            and load_native(False)):     # a process that built only another kernel group keeps the vendor GEMM
         if out is None:
             out = torch.empty(M, N, dtype=x.dtype, device=x.device)
         _call("skinny_gemm", out, x, w, bias, _skinny_cfg(M, N))

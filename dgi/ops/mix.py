@@ -210,6 +210,47 @@ def masked_attn_rows(q, k_cache, v_cache, block_tables, cu_seqlens, positions, H
 
 
 # ----------------------------------------------------------------------------
+# MFMA prompt attention with a block mask (bf16, equal key / value size of 64 or 128)
+# ----------------------------------------------------------------------------
+
+MASKED_PREFILL = os.environ.get("DGI_MASKED_PREFILL", "1") == "1"   # 0: prompt rows on the row-wise kernel (A/B)
+
+
+def masked_prefill_available() -> bool:
+    """Whether prompt portions may take the MFMA kernel with a block mask and gate epilogue."""
+    from dgi import ops
+    return MASKED_PREFILL and ops.PREFILL_TILE == 128
+
+
+def paged_prefill_masked(q, k_cache, v_cache, block_tables, cu_seqlens_q, context_lens, nh, nkv, scale,
+                         mask: int = 0, gate=None, tiles=None, out=None) -> torch.Tensor:
+    """``paged_prefill`` with a block mask — a query at position p sees keys
+    [floor(p / mask) * mask, p] (``mask`` 0: all keys up to p) — and an optional sigmoid output
+    gate (out *= sigmoid(gate)).  bf16, key size == value size in {64, 128} on the GPU
+    (dgi/csrc/mix/masked_prefill.hip); the row-wise reference elsewhere."""
+    from dgi import ops
+    if _native(q):
+        hd = k_cache.shape[-1]
+        if out is None:
+            out = torch.empty(q.shape[0], nh * hd, dtype=q.dtype, device=q.device)
+        if tiles is None:
+            tl = ops.prefill_tiles(cu_seqlens_q.tolist(), context_lens=context_lens.tolist(), tile=128)
+            tiles = torch.tensor(tl if tl else [[0, 0]], dtype=torch.int32, device=q.device)[: len(tl)]
+        _call("paged_prefill_masked", out, q, k_cache, v_cache, block_tables, cu_seqlens_q, context_lens, tiles,
+              nh, nkv, float(scale), int(mask), gate)
+        return out
+    cu = cu_seqlens_q.tolist()
+    pos = torch.cat([torch.arange(int(context_lens[b]) - (cu[b + 1] - cu[b]), int(context_lens[b]), dtype=torch.int32)
+                     for b in range(len(cu) - 1)]) if len(cu) > 1 else torch.zeros(0, dtype=torch.int32)
+    r = masked_attn_rows_ref(q, k_cache, v_cache, block_tables, cu_seqlens_q, pos.to(q.device), nh, nkv, scale,
+                             mask, gate)
+    if out is not None:
+        out.copy_(r)
+        return out
+    return r
+
+
+# ----------------------------------------------------------------------------
 # Activations / logits
 # ----------------------------------------------------------------------------
 

@@ -261,7 +261,7 @@ def test_masked_prefill_mfma_edges(hd):
         cu = torch.tensor([0, ql], dtype=torch.int32).to(dev)
         cl = torch.tensor([ctx], dtype=torch.int32).to(dev)
         args = (q.reshape(ql, -1).to(dev), kc.to(dev), vc.to(dev), bt.to(dev), cu)
-        out = ops.paged_prefill_masked(*args, cl, H, G, 0.2, chunk, gate.to(dev)).cpu()
+        out = mix.paged_prefill_masked(*args, cl, H, G, 0.2, chunk, gate.to(dev)).cpu()
         pos = torch.arange(ctx - ql, ctx, dtype=torch.int32).to(dev)
         rows = mix.masked_attn_rows(*args, pos, H, G, 0.2, chunk, gate.to(dev)).cpu()
         close(out, rows, 0.3)
@@ -400,11 +400,11 @@ def test_mfma_prompt_path_in_the_model():
     mk = lambda: engine(cfg, "cuda", torch.bfloat16, num_blocks=64, bs=16, max_len=512)     # noqa: E731
     a = feed_all(mk(), "a", t, [300])
     b = feed_all(mk(), "b", t, [130, 2, 77, 64])
-    ops.MASKED_PREFILL = False
+    mix.MASKED_PREFILL = False
     try:
         c = feed_all(mk(), "c", t, [300])
     finally:
-        ops.MASKED_PREFILL = True
+        mix.MASKED_PREFILL = True
     want = oracle_logits(engine(cfg, "cpu", torch.bfloat16, bs=16, num_blocks=8), t[:80])[0]
     scale = want.std().item()
     rms = lambda x, y: (x.double() - y.double()).pow(2).mean().sqrt().item()      # noqa: E731
