@@ -412,6 +412,59 @@ def test_mfma_prompt_path_in_the_model():
     assert rms(a[:80], want) < 0.06 * scale
 
 
+def _layer(H, G, dk, dv, rd, chunk, ff, sc=None, base=10000.0, lim=1.2):
+    return LayerSpec("attention", AttentionSpec(H, G, dk, dv, dk ** -0.5, RotarySpec(base, rd, sc), "chunk", chunk),
+                     GluSpec(ff, lim) if ff else None)
+
+
+_SC = {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 32}
+GEOMETRIES = {
+    # heads of 64 and 128 (the MFMA prompt kernel in bf16 on a GPU) under block sizes that are no multiple of a
+    # page or a key tile; a block longer than any sequence; a rotary of one pair
+    "equal-64-128-odd-blocks": (96, 128, [_layer(4, 2, 64, 64, 32, 37, 160, _SC), _layer(2, 1, 128, 128, 128, 50, 0),
+                                          _layer(8, 1, 64, 64, 2, 1000, 96)]),
+    # 8 and 16 query heads per kv head, key size != value size, sizes that are multiples of 8 but not of 16
+    "wide-groups": (70, 64, [_layer(8, 1, 32, 16, 16, 9, 64), _layer(16, 1, 16, 32, 8, 20, 0, _SC),
+                             _layer(6, 3, 96, 40, 48, 33, 72)]),
+    # a block of ONE position (every token sees only itself), a width that is no multiple of 4, odd-ish head sizes
+    "block-of-one": (33, 50, [_layer(2, 1, 36, 12, 36, 1, 30), _layer(2, 2, 10, 6, 4, 3, 0), _layer(1, 1, 64, 128, 64, 64, 20)]),
+    "wide-heads": (50, 256, [_layer(2, 1, 256, 256, 64, 24, 512, _SC, 500000.0), _layer(4, 4, 128, 64, 128, 17, 0)]),
+    "no-feed-forward": (40, 64, [_layer(4, 2, 16, 16, 16, 11, 0), _layer(4, 1, 8, 24, 8, 40, 0)]),
+}
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, 3e-5), (torch.bfloat16, 0.06)])
+@pytest.mark.parametrize("name", list(GEOMETRIES))
+def test_other_geometries_mixed_batches(device, dtype, tol, name):
+    """Sizes, head ratios, block sizes and layer orders unlike the small configuration's, each run
+    as three unequal requests in mixed steps (portions beside decode rows, pages reused) in a pool
+    of 13 pages of 16 tokens, against the oracle."""
+    vocab, W, layers = GEOMETRIES[name]
+    cfg = BebovikConfig(name="g", vocab_size=vocab, hidden_size=W, layers=layers, embedding_scale=2.5, logit_scale=0.7,
+                        logit_softcap=9.0, norm_eps=1e-5, max_position=512)
+    eng = engine(cfg, device, dtype, num_blocks=14, bs=16, seed=11, max_len=192)
+    seqs = {"a": toks(75, 70, vocab), "b": toks(31, 71, vocab), "c": toks(58, 72, vocab)}
+    P, C = orc.from_model(eng.model)
+    got, at = {k: [] for k in seqs}, {k: 0 for k in seqs}
+    plan = [({"a": 40}, []), ({"a": 1, "b": 2}, []), ({"a": 1, "b": 1, "c": 17}, []), ({"a": 30, "b": 27, "c": 1}, []),
+            ({"a": 1, "b": 1, "c": 2}, ["b"]), ({"a": 1, "c": 37}, []), ({"a": 1, "c": 1}, ["a", "c"])]
+    for entries, end in plan:
+        batch = []
+        for k, n in entries.items():
+            part = seqs[k][at[k]:at[k] + n]
+            batch.append((k, part, list(range(len(part)))))
+            at[k] += n
+        for (k, _p, _w), lg in zip(batch, eng.feed(batch, end)):
+            got[k].append(lg)
+    for k, t in seqs.items():
+        assert at[k] == len(t)
+        want = orc.forward(t, P, C)[0]
+        d = torch.cat(got[k], 0).double() - want
+        d = d - d.mean(-1, keepdim=True)
+        assert (d.pow(2).mean(-1).sqrt() / want.std()).max().item() < tol
+
+
 # ----------------------------------------------------------------------------------- files, CLI
 def _design_json(cfg: BebovikConfig) -> dict:
     lay = []
