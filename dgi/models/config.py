@@ -322,7 +322,7 @@ PRESETS: dict[str, ModelConfig] = {
                             rms_eps=1.5625e-07, max_position=4096, qkv_bias=True, rotary_dim=64,
                             rope_interleaved=True, bos_token_id=1, eos_token_id=2),
     # Bebovik test / smoke sizes (random weights): chunk-masked GQA attention, half-rotary heads
-    "bebovik-tiny": bebovik_uniform("bebovik-tiny", 1024, 256, 3, 4, 2, 64, 64, 512, 48, rot_dims=32,
+    "bebovik-tiny": bebovik_uniform("bebovik-tiny", 1024, 256, 3, 4, 2, 64, 64, 512, 48, rot_dims=16,
                                     embedding_scale=4.0, logit_scale=0.5, logit_softcap=30.0, max_position=4096,
                                     bos_token_id=1, eos_token_id=2),
     "opt-125m": ModelConfig(name="opt-125m", arch="opt", vocab_size=50272, hidden_size=768,

@@ -275,12 +275,12 @@ def test_masked_prefill_mfma_edges(hd):
 def test_glu_and_softcap(device, dtype):
     g = torch.Generator().manual_seed(4)
     gu = (torch.randn(3, 2 * 37, generator=g) * 4).to(dtype)           # both clamps active
-    lim = 1.5
+    lim = 1.3
     a, u = gu[:, :37].double().clamp(max=lim), gu[:, 37:].double().clamp(-lim, lim)
     want = a * torch.sigmoid(1.702 * a) * (u + 1)
     close(mix.glu_clamped(gu.to(device), lim).cpu(), want, 1e-5 if dtype == torch.float32 else 3e-2)
     x = (torch.randn(2, 50, generator=g) * 20).to(dtype)
-    close(mix.scale_softcap(x.to(device), 2.0, 15.0).cpu(), 15.0 * torch.tanh(x.double() * 2.0 / 15.0), 1e-4)
+    close(mix.scale_softcap(x.to(device), 1.7, 11.0).cpu(), 11.0 * torch.tanh(x.double() * 1.7 / 11.0), 1e-4)
     close(mix.scale_softcap(x.to(device), 0.5, 0.0).cpu(), x.double() * 0.5, 1e-5)
 
 
@@ -594,3 +594,15 @@ def test_prefix_cache_hit_generates_the_same_tokens(device):
     assert c.output == a.output
     fresh = engine(cfg, device)
     assert fresh.generate([p + [5, 6]], sp)[0].output == b.output
+
+
+def test_bench_arch_compare_option_runs():
+    """`bench.py --arch-compare` (tiny size, CPU): one JSON line with a row per model and phase numbers."""
+    r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--arch-compare", "bebovik", "--arch-sizes", "tiny",
+                        "--prompt-len", "40", "--concurrency", "2", "--steps", "2", "--warmup", "1",
+                        "--max-batched-tokens", "128"], capture_output=True, text=True, timeout=600,
+                       env={**os.environ, "CUDA_VISIBLE_DEVICES": "", "HIP_VISIBLE_DEVICES": ""})
+    assert r.returncode == 0, r.stderr[-2000:]
+    out = json.loads(r.stdout.strip().splitlines()[-1])
+    assert [x["model"] for x in out["rows"]] == ["bebovik", "llama"]
+    assert all(x["prefill_tok_s"] > 0 and x["decode_tok_s"] > 0 for x in out["rows"])
