@@ -110,7 +110,8 @@ class BebovikModel:
             L = BebovikLayerWeights()
             L.spec = spec
             L.norm1, L.norm1b = self._norm(W), self._norm(W)
-            L.qkvg = torch.empty(m.q_size + m.k_size + m.v_size + m.o_size, W, device=dev, dtype=dt)
+            gate_rows = m.o_size if m.out_gate else 0
+            L.qkvg = torch.empty(m.q_size + m.k_size + m.v_size + gate_rows, W, device=dev, dtype=dt)
             L.o = torch.empty(W, m.o_size, device=dev, dtype=dt)
             L.q_norm = torch.ones(m.dim, device=dev)
             L.k_norm = torch.ones(m.dim, device=dev)

@@ -144,8 +144,7 @@ class AttentionSpec:
     rot: Optional[RotarySpec] = None
     mask_kind: str = "causal"
     mask_size: int = 0
-    qk_norm: bool = True
-    out_gate: bool = True
+    out_gate: bool = True        # sigmoid(W_g h) on the concatenated heads before the output projection
 
     @property
     def q_size(self) -> int:

@@ -198,8 +198,9 @@ def load_bebovik_checkpoint(model, path: str) -> dict:
         m = L.spec.mixer
         p = f"l{li}."
         r = 0
-        for key, rows in (("q", m.q_size), ("k", m.k_size), ("v", m.v_size), ("g", m.o_size)):
-            put(L.qkvg[r:r + rows], p + "mix." + key)
+        for key, rows in (("q", m.q_size), ("k", m.k_size), ("v", m.v_size), ("g", m.o_size if m.out_gate else 0)):
+            if rows:
+                put(L.qkvg[r:r + rows], p + "mix." + key)
             r += rows
         put(L.o, p + "mix.o")
         put(L.q_norm, p + "mix.q.norm")

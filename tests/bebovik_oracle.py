@@ -80,7 +80,9 @@ def attention_mixer(h, p, m, eps, pos0=0):
             s = torch.stack([(q[i, hh] * k[j, g]).sum() * m["scale"] for j in keys])
             w = torch.softmax(s, 0)
             o[i, hh] = sum(w[n] * v[j, g] for n, j in enumerate(keys))
-    o = o.reshape(T, H * dv) * torch.sigmoid(h @ p["g"].to(F64).T)
+    o = o.reshape(T, H * dv)
+    if p["g"].numel():                      # output gate from the mixer's own input
+        o = o * torch.sigmoid(h @ p["g"].to(F64).T)
     return o @ p["o"].to(F64).T
 
 

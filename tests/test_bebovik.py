@@ -417,6 +417,11 @@ def _layer(H, G, dk, dv, rd, chunk, ff, sc=None, base=10000.0, lim=1.2):
                      GluSpec(ff, lim) if ff else None)
 
 
+def _ungated(layer):
+    layer.mixer.out_gate = False
+    return layer
+
+
 _SC = {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 32}
 GEOMETRIES = {
     # heads of 64 and 128 (the MFMA prompt kernel in bf16 on a GPU) under block sizes that are no multiple of a
@@ -430,6 +435,8 @@ GEOMETRIES = {
     "block-of-one": (33, 50, [_layer(2, 1, 36, 12, 36, 1, 30), _layer(2, 2, 10, 6, 4, 3, 0), _layer(1, 1, 64, 128, 64, 64, 20)]),
     "wide-heads": (50, 256, [_layer(2, 1, 256, 256, 64, 24, 512, _SC, 500000.0), _layer(4, 4, 128, 64, 128, 17, 0)]),
     "no-feed-forward": (40, 64, [_layer(4, 2, 16, 16, 16, 11, 0), _layer(4, 1, 8, 24, 8, 40, 0)]),
+    "no-output-gate": (40, 64, [_ungated(_layer(4, 2, 16, 16, 8, 11, 48)), _layer(2, 1, 64, 64, 64, 40, 0),
+                                _ungated(_layer(2, 1, 64, 64, 32, 23, 0))]),
 }
 
 
