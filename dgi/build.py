@@ -66,6 +66,9 @@ def build(verbose: bool = False, force: bool = False, group: str = "core") -> st
     hdrs = [os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith(".h")]
     hdrs += [os.path.join(src_dir, f) for f in os.listdir(src_dir) if f.endswith(".h") and src_dir != CSRC]
     kernels = sorted(f for f in os.listdir(src_dir) if f.endswith(".hip"))
+    sources = [os.path.join(src_dir, f) for f in os.listdir(src_dir) if f.endswith((".hip", ".cpp", ".cc"))]
+    if not force and not _newer(sources + hdrs, out):
+        return out      # the library is newer than every source (object files need not travel with it)
     common = ["-O3", "-fPIC", "-std=c++17", f"-D_GLIBCXX_USE_CXX11_ABI={abi}"]
     jobs = []
     objs = []
