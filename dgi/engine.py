@@ -477,8 +477,10 @@ class LLMEngine:
         named = {}
         for rid, toks, want in entries:
             toks = [int(t) for t in toks]
-            if not toks or rid in named:
-                raise ValueError("feed(): every entry brings tokens, one entry per request and step")
+            if rid in named:
+                raise ValueError("feed(): one entry per request and step")
+            if not toks:            # an entry without tokens asks for nothing and changes nothing
+                continue
             req = self.requests.get(rid)
             if req is None:
                 req = Request(toks, SamplingParams(max_tokens=1 << 30, temperature=0.0, ignore_eos=True), rid=rid)
@@ -508,8 +510,11 @@ class LLMEngine:
                 raise RuntimeError(f"feed(): request {rid!r} did not fit this step (pool pages or token budget)")
             if c is not None:
                 c.logit_pos = want
-        logits = self.runner.execute_logits(sb)
-        self._advance(sb)
+        if sb.empty:                # a step that only ends requests
+            logits = torch.zeros(0, self.model_cfg.vocab_size)
+        else:
+            logits = self.runner.execute_logits(sb)
+            self._advance(sb)
         out = []
         row = len(sb.decode)
         first = {}
@@ -517,6 +522,9 @@ class LLMEngine:
             first[c.req.rid] = row
             row += len(c.logit_pos or ())
         for rid, _toks, _want in entries:
+            if rid not in named:
+                out.append(logits[:0])
+                continue
             req, n, want = named[rid]
             if rid in dec_row:
                 out.append(logits[dec_row[rid]: dec_row[rid] + 1] if want else logits[:0])
