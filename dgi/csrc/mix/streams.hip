@@ -1,0 +1,190 @@
+// dgi/csrc/mix/streams.hip — several fp32 residual streams per token ("hyper-connections") and the
+// embedding that starts them.
+//
+//   embed_streams   x_s[t] = E[tok] + Bg[(prev * a + tok * b) mod n] + P[pos]  for every stream s
+//                   (a sequence's first token takes bigram row n; the token before a portion's first
+//                   row comes from the sequence's state slot, which then receives the portion's last
+//                   token in a second, tiny kernel — a portion's first and last rows are different
+//                   workgroups, so the slot is not rewritten while it may still be read)
+//   hc_mix_norm     one pass over a token's S streams that (a) applies the update of the sublayer
+//                   that just ran, x_t <- sum_s mix[s][t] x_s + out[t] * y * sigmoid(gate + gate_b),
+//                   all streams from the old values, and (b) reads the next sublayer's input out of the
+//                   new values, u = sum_s in[s] x_s, h = (u - mean) / sqrt(var + eps) * w, written in
+//                   fp32 and, for bf16 models, also in bf16 (the GEMM input).  Either half may be absent.
+//
+// All arithmetic is fp32; the variance is the mean of squared deviations (two passes over the row,
+// which sits in LDS).  One workgroup per token row.
+#include "../common.h"
+
+using namespace dgi;
+
+namespace {
+
+template <typename T> __device__ __forceinline__ float ldf(const T* p);
+template <> __device__ __forceinline__ float ldf<float>(const float* p) { return *p; }
+template <> __device__ __forceinline__ float ldf<uint16_t>(const uint16_t* p) { return bf16_to_f32(*p); }
+
+constexpr int MAXS = 8;      // streams
+
+__device__ __forceinline__ float block_sum(float v, float* red) {
+  v = wave_sum(v);
+  const int w = threadIdx.x >> 6, nw = blockDim.x >> 6;
+  __syncthreads();
+  if ((threadIdx.x & 63) == 0) red[w] = v;
+  __syncthreads();
+  float r = 0.f;
+  for (int i = 0; i < nw; ++i) r += red[i];
+  return r;
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void embed_streams_kernel(
+    float* __restrict__ xs, int S, int T, int W, const int* __restrict__ ids, const int* __restrict__ positions,
+    const int* __restrict__ row_seq, const int* __restrict__ seq_row0, const int* __restrict__ seq_slots,
+    const int* __restrict__ prev_tok, const T* __restrict__ embed, int vocab, const T* __restrict__ bigram,
+    int buckets, long long mul_prev, long long mul_cur, const T* __restrict__ pos_table, int max_pos) {
+  const int row = blockIdx.x;
+  int tok = ids[row];
+  tok = tok < 0 ? 0 : (tok >= vocab ? vocab - 1 : tok);
+  const int pos = positions[row];
+  const T* e = embed + (size_t)tok * W;
+  const T* b = nullptr;
+  if (bigram) {
+    long long br = buckets;
+    if (pos > 0) {
+      const int seq = row_seq[row];
+      const long long prev = row == seq_row0[seq] ? prev_tok[seq_slots[seq]] : ids[row - 1];
+      br = (prev * mul_prev + (long long)ids[row] * mul_cur) % buckets;
+      if (br < 0) br += buckets;
+    }
+    b = bigram + (size_t)br * W;
+  }
+  const T* p = nullptr;
+  if (pos_table) p = pos_table + (size_t)(pos < 0 ? 0 : (pos >= max_pos ? max_pos - 1 : pos)) * W;
+  for (int w = threadIdx.x; w < W; w += blockDim.x) {
+    float v = ldf<T>(e + w);
+    if (b) v += ldf<T>(b + w);
+    if (p) v += ldf<T>(p + w);
+    for (int s = 0; s < S; ++s) xs[((size_t)s * T + row) * W + w] = v;
+  }
+}
+
+__global__ void store_last_token_kernel(int* __restrict__ prev_tok, const int* __restrict__ ids,
+                                        const int* __restrict__ seq_row0, const int* __restrict__ seq_slots, int n) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  const int r0 = seq_row0[i], r1 = seq_row0[i + 1];
+  if (r1 > r0) prev_tok[seq_slots[i]] = ids[r1 - 1];
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void hc_mix_norm_kernel(
+    float* __restrict__ xs, int S, int T, int W, const T* __restrict__ y, int y_stride, const T* __restrict__ gate,
+    int gate_stride, const float* __restrict__ gate_b, const float* __restrict__ mixm, const float* __restrict__ outc,
+    const float* __restrict__ in_next, const float* __restrict__ norm_w, float eps, float* __restrict__ h32,
+    T* __restrict__ hd) {
+  extern __shared__ float us[];          // [W] the read-out row
+  __shared__ float red[8];
+  __shared__ float cm[MAXS * MAXS], co[MAXS], ci[MAXS];
+  const int row = blockIdx.x;
+  if (threadIdx.x < S * S && y) cm[threadIdx.x] = mixm[threadIdx.x];
+  if (threadIdx.x < S) {
+    if (y) co[threadIdx.x] = outc[threadIdx.x];
+    if (in_next) ci[threadIdx.x] = in_next[threadIdx.x];
+  }
+  __syncthreads();
+  float sum = 0.f;
+  for (int w = threadIdx.x; w < W; w += blockDim.x) {
+    float x[MAXS];
+#pragma unroll
+    for (int s = 0; s < MAXS; ++s) x[s] = s < S ? xs[((size_t)s * T + row) * W + w] : 0.f;
+    if (y) {
+      float yy = ldf<T>(y + (size_t)row * y_stride + w);
+      if (gate) yy *= 1.f / (1.f + expf(-(ldf<T>(gate + (size_t)row * gate_stride + w) + gate_b[w])));
+      float nx[MAXS];
+#pragma unroll
+      for (int t = 0; t < MAXS; ++t) {
+        float a = 0.f;
+        if (t < S) {
+#pragma unroll
+          for (int s = 0; s < MAXS; ++s)
+            if (s < S) a += cm[s * S + t] * x[s];
+          a += co[t] * yy;
+          xs[((size_t)t * T + row) * W + w] = a;
+        }
+        nx[t] = a;
+      }
+#pragma unroll
+      for (int t = 0; t < MAXS; ++t) x[t] = nx[t];
+    }
+    if (in_next) {
+      float u = 0.f;
+#pragma unroll
+      for (int s = 0; s < MAXS; ++s)
+        if (s < S) u += ci[s] * x[s];
+      us[w] = u;
+      sum += u;
+    }
+  }
+  if (!in_next) return;
+  const float mean = block_sum(sum, red) / (float)W;
+  float sq = 0.f;
+  for (int w = threadIdx.x; w < W; w += blockDim.x) {
+    const float d = us[w] - mean;
+    sq += d * d;
+  }
+  const float rstd = 1.f / sqrtf(block_sum(sq, red) / (float)W + eps);
+  for (int w = threadIdx.x; w < W; w += blockDim.x) {
+    const float h = (us[w] - mean) * rstd * norm_w[w];
+    h32[(size_t)row * W + w] = h;
+    if constexpr (sizeof(T) == 2) {
+      if (hd) hd[(size_t)row * W + w] = f32_to_bf16(h);
+    }
+  }
+}
+
+}  // namespace
+
+extern "C" int dgi_embed_streams(float* xs, int S, int T, int W, const int* ids, const int* positions,
+                                 const int* row_seq, const int* seq_row0, const int* seq_slots, int n_seq,
+                                 int* prev_tok, const void* embed, int vocab, const void* bigram, int buckets,
+                                 long long mul_prev, long long mul_cur, const void* pos_table, int max_pos, int is_f32,
+                                 hipStream_t s) {
+  if (T == 0) return 0;
+  if (S < 1 || S > MAXS) return -2;
+  if (bigram && buckets <= 0) return -3;
+  if (is_f32)
+    embed_streams_kernel<float><<<T, 256, 0, s>>>(xs, S, T, W, ids, positions, row_seq, seq_row0, seq_slots, prev_tok,
+                                                  (const float*)embed, vocab, (const float*)bigram, buckets, mul_prev,
+                                                  mul_cur, (const float*)pos_table, max_pos);
+  else
+    embed_streams_kernel<uint16_t><<<T, 256, 0, s>>>(xs, S, T, W, ids, positions, row_seq, seq_row0, seq_slots,
+                                                     prev_tok, (const uint16_t*)embed, vocab, (const uint16_t*)bigram,
+                                                     buckets, mul_prev, mul_cur, (const uint16_t*)pos_table, max_pos);
+  DGI_CHECK_LAUNCH();
+  store_last_token_kernel<<<(n_seq + 255) / 256, 256, 0, s>>>(prev_tok, ids, seq_row0, seq_slots, n_seq);
+  DGI_CHECK_LAUNCH();
+  return 0;
+}
+
+// y / gate: bf16 (is_f32 0) or fp32 rows with their own strides, or null; hd: bf16 copy of h (bf16 models)
+extern "C" int dgi_hc_mix_norm(float* xs, int S, int T, int W, const void* y, int y_stride, const void* gate,
+                               int gate_stride, const float* gate_b, const float* mixm, const float* outc,
+                               const float* in_next, const float* norm_w, float eps, float* h32, void* hd, int is_f32,
+                               hipStream_t s) {
+  if (T == 0) return 0;
+  if (S < 1 || S > MAXS) return -2;
+  if (W > 16384) return -3;
+  const size_t lds = in_next ? (size_t)W * 4 : 0;
+  if (is_f32) {
+    if (hd) return -4;
+    hc_mix_norm_kernel<float><<<T, 256, lds, s>>>(xs, S, T, W, (const float*)y, y_stride, (const float*)gate,
+                                                  gate_stride, gate_b, mixm, outc, in_next, norm_w, eps, h32, nullptr);
+  } else {
+    hc_mix_norm_kernel<uint16_t><<<T, 256, lds, s>>>(xs, S, T, W, (const uint16_t*)y, y_stride, (const uint16_t*)gate,
+                                                     gate_stride, gate_b, mixm, outc, in_next, norm_w, eps, h32,
+                                                     (uint16_t*)hd);
+  }
+  DGI_CHECK_LAUNCH();
+  return 0;
+}

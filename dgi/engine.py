@@ -133,12 +133,24 @@ class LLMEngine:
             shapes = mc.kv_layer_shapes(self.model.layer_start, self.model.layer_end) or None
         self.pool = BlockPool(nblocks, cfg.block_size, max(1, n_local), mc.num_kv_heads, mc.head_dim,
                               cfg.dtype, self.device, layer_shapes=shapes)
+        # per-sequence state slots of models that carry more than pages (dgi.kv.state_pool); such a
+        # sequence cannot resume from shared prefix pages or host-tier pages alone, so neither is on
+        self.state_pool = None
+        prefix = cfg.enable_prefix_caching
+        if hasattr(self.model, "state_fields"):
+            from dgi.kv.state_pool import StatePool
+            if cfg.host_kv_gb > 0:
+                raise ValueError("the host KV tier does not hold per-sequence state; host_kv_gb must be 0 for this model")
+            self.state_pool = StatePool(cfg.max_num_seqs, self.model.state_fields(), self.device)
+            prefix = False
         align = cfg.token_align if cfg.token_align >= 0 else (256 if self.device.type == "cuda" else 0)
         self.scheduler = Scheduler(self.pool, SchedulerConfig(cfg.max_num_seqs, cfg.max_num_batched_tokens,
-                                                              cfg.max_model_len, cfg.enable_prefix_caching,
-                                                              token_align=align))
+                                                              cfg.max_model_len, prefix, token_align=align))
+        self.scheduler.state_pool = self.state_pool
         self.host_tier = None
         host_gb = cfg.host_kv_gb
+        if host_gb < 0 and self.state_pool is not None:
+            host_gb = 0.0
         if host_gb < 0:      # auto: GPU engines only (CPU rehearsals have no HBM to relieve)
             host_gb = auto_host_kv_gb(self.pool, self.device) if self.device.type == "cuda" else 0.0
         if host_gb > 0:
@@ -147,11 +159,11 @@ class LLMEngine:
             cap = max(1, int(host_gb * (1 << 30) // self.pool.page_bytes()))
             self.host_tier = HostKVTier(self.pool, cap)
             self.scheduler.host_tier = self.host_tier
-            if cfg.enable_prefix_caching:
+            if prefix:
                 self.scheduler.radix = RadixCache(self.pool, self.host_tier)
         rkw = {"graph_buckets": tuple(cfg.graph_buckets)} if cfg.graph_buckets else {}
         self.runner = ModelRunner(self.model, self.pool, cfg.max_num_seqs, cfg.max_model_len,
-                                  cfg.max_num_batched_tokens, cfg.use_graphs, **rkw)
+                                  cfg.max_num_batched_tokens, cfg.use_graphs, state_pool=self.state_pool, **rkw)
         self.runner.host_tier = self.host_tier
         self.requests: dict = {}
         # decode lookahead: (ScheduledBatch, launch handle) of a step in flight, not applied yet
@@ -261,7 +273,7 @@ class LLMEngine:
             self._account(n, time.perf_counter() - t0)
             return outs
         if hasattr(self.model, "attach_cache"):   # engines may share one model object
-            self.model.attach_cache(self.pool)
+            self._attach()
         else:
             self.model.kv_cache = self.pool.kv
         with phase("schedule"):
@@ -297,6 +309,12 @@ class LLMEngine:
         if sbud is not None and sb.prefill:       # mixed / prefill steps set the per-row cost
             sbud.observe(sb.num_tokens, dt * 1e3)
         return outs
+
+    def _attach(self) -> None:
+        if self.state_pool is not None:
+            self.model.attach_cache(self.pool, self.state_pool)
+        else:
+            self.model.attach_cache(self.pool)
 
     def _account(self, rows: int, dt: float) -> None:
         """Step wall time and row-count histogram (every step, lookahead chains included)."""
@@ -497,7 +515,7 @@ class LLMEngine:
             r.busy = r.rid not in named
         try:
             if hasattr(self.model, "attach_cache"):
-                self.model.attach_cache(self.pool)
+                self._attach()
             sb = sch.schedule(preempt=False)
         finally:
             for r in sch.running:

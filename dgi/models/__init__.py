@@ -1,4 +1,4 @@
-from dgi.models.config import BebovikConfig, ModelConfig, PRESETS, get_config  # noqa: F401
+from dgi.models.config import BebovikConfig, ModelConfig, PRESETS, TifepelConfig, get_config  # noqa: F401
 
 
 def model_class(cfg):
@@ -6,6 +6,9 @@ def model_class(cfg):
     if isinstance(cfg, BebovikConfig):
         from dgi.models.bebovik import BebovikModel
         return BebovikModel
+    if isinstance(cfg, TifepelConfig):
+        from dgi.models.tifepel import TifepelModel
+        return TifepelModel
     from dgi.models.llama import LlamaModel
     return LlamaModel
 

@@ -145,6 +145,14 @@ class AttentionSpec:
     mask_kind: str = "causal"
     mask_size: int = 0
     out_gate: bool = True        # sigmoid(W_g h) on the concatenated heads before the output projection
+    qk_norm_weight: bool = True  # learned per-dim weight after the q / k unit-RMS norm
+    # query temperature: q *= 1 + coef * ln(floor((p + 1) / every) + 1) at position p (every 0: none)
+    q_temp_coef: float = 0.0
+    q_temp_every: int = 0
+    # learned distance bias added to the scaled scores: a table [bias_rows, heads] indexed by
+    # ``distance_bucket(i - j, bias_rows, bias_max)`` (bias_rows 0: none)
+    bias_rows: int = 0
+    bias_max: float = 0.0
 
     @property
     def q_size(self) -> int:
@@ -171,11 +179,65 @@ class GluSpec:
     kind: str = "dense"
 
 
+def distance_bucket(n: int, rows: int, far: float) -> int:
+    """Row of a distance-bias table for distance ``n`` >= 0: the first ``rows // 2`` distances have
+    a row each, the rest share rows on a logarithmic scale that reaches the last row at ``far``."""
+    import math
+    half = rows // 2
+    if n < half:
+        return n
+    return min(rows - 1, half + int(math.floor(math.log(n / half) / math.log(far / half) * (rows - half))))
+
+
+@dataclasses.dataclass
+class Mamba2Spec:
+    """One Mamba-2 (state-space duality) mixer: ``heads`` heads of ``vdim`` channels share
+    ``groups`` B / C projections of ``state`` dims; a causal convolution of ``conv`` taps over
+    x | B | C; the gated output is RMS-normed in ``norm_groups`` equal parts."""
+    heads: int
+    vdim: int
+    state: int
+    groups: int
+    conv: int
+    norm_groups: int = 1
+
+    @property
+    def inner(self) -> int:
+        return self.heads * self.vdim
+
+    @property
+    def conv_channels(self) -> int:
+        return self.inner + 2 * self.groups * self.state
+
+    @property
+    def in_size(self) -> int:
+        """Rows of the input projection: z | x | B | C | dt."""
+        return 2 * self.inner + 2 * self.groups * self.state + self.heads
+
+
+@dataclasses.dataclass
+class MoeSpec:
+    """Mixture-of-experts feed-forward: ``experts`` gated-SiLU experts of width ``ff`` plus
+    ``identity`` experts that return their input; a token takes the ``top`` experts with the
+    largest softmax score + selection bias and weighs them by the plain scores (not
+    renormalised).  ``shared_ff`` > 0: a shared expert of that width runs for every token."""
+    experts: int
+    identity: int
+    top: int
+    ff: int
+    shared_ff: int = 0
+    kind: str = "moe"
+
+    @property
+    def routes(self) -> int:
+        return self.experts + self.identity
+
+
 @dataclasses.dataclass
 class LayerSpec:
     type: str
-    mixer: AttentionSpec
-    mlp: Optional[GluSpec] = None
+    mixer: object                     # AttentionSpec | Mamba2Spec
+    mlp: Optional[object] = None      # GluSpec | MoeSpec
 
 
 @dataclasses.dataclass
@@ -278,7 +340,157 @@ def bebovik_uniform(name: str, vocab: int, width: int, n_layers: int, heads: int
     return BebovikConfig(name=name, vocab_size=vocab, hidden_size=width, layers=[layer() for _ in range(n_layers)], **kw)
 
 
-NATIVE_CONFIGS = {"bebovik": BebovikConfig.from_dict}
+@dataclasses.dataclass
+class TifepelConfig:
+    """A Tifepel decoder: token + hashed-bigram + learned-position embedding, ``streams``
+    hyper-connected residual streams, per-layer attention (distance-biased, no rotation) or
+    Mamba-2 mixers, mixture-of-experts feed-forwards, a causal input convolution and a sigmoid
+    output gate around every sublayer, and a span of layers run several times with the same
+    weights (``loop_start`` .. ``loop_stop`` - 1, ``loop_times`` times; every pass has its own
+    cache and state)."""
+    name: str
+    vocab_size: int
+    hidden_size: int
+    layers: list
+    streams: int = 1
+    canon_taps: int = 0
+    bigram_buckets: int = 0
+    bigram_mul_prev: int = 0
+    bigram_mul_cur: int = 0
+    loop_start: int = 0
+    loop_stop: int = 0
+    loop_times: int = 1
+    norm_eps: float = 1e-6
+    max_position: int = 2048
+    bos_token_id: int = -1
+    eos_token_id: int = -1
+    arch: str = "tifepel"
+    tie_embeddings: bool = False
+
+    @property
+    def num_layers(self) -> int:
+        return len(self.layers)
+
+    @property
+    def layer_runs(self) -> list:
+        """Layer index of every layer run, in execution order."""
+        n = len(self.layers)
+        if self.loop_times == 1 or self.loop_stop <= self.loop_start:
+            return list(range(n))
+        a, b = self.loop_start, self.loop_stop
+        return list(range(a)) + list(range(a, b)) * self.loop_times + list(range(b, n))
+
+    def _attn(self):
+        return [l.mixer for l in self.layers if l.type == "attention"]
+
+    @property
+    def num_heads(self) -> int:
+        return max([m.heads for m in self._attn()] or [1])
+
+    @property
+    def num_kv_heads(self) -> int:
+        return max([m.kv_heads for m in self._attn()] or [1])
+
+    @property
+    def head_dim(self) -> int:
+        return max([max(m.dim, m.vdim) for m in self._attn()] or [1])
+
+    @property
+    def rms_eps(self) -> float:
+        return self.norm_eps
+
+    def kv_layer_shapes(self, start: int = 0, end: Optional[int] = None) -> list:
+        """(kv heads, key size, value size) of the cache pages of every attention layer RUN
+        (a looped layer has pages per pass); Mamba-2 runs hold no pages."""
+        out = []
+        for li in self.layer_runs:
+            l = self.layers[li]
+            if l.type == "attention":
+                out.append((l.mixer.kv_heads, l.mixer.dim, l.mixer.vdim))
+        return out
+
+    def kv_bytes_per_token(self, dtype_bytes: int = 2, layers: Optional[int] = None) -> int:
+        return sum(g * (dk + dv) for g, dk, dv in self.kv_layer_shapes()) * dtype_bytes
+
+    def param_count(self) -> int:
+        W = self.hidden_size
+        n = 2 * self.vocab_size * W + (self.bigram_buckets + 1) * W + self.max_position * W
+        for l in self.layers:
+            m = l.mixer
+            if l.type == "attention":
+                n += W * (m.q_size + m.k_size + m.v_size) + m.o_size * W
+            else:
+                n += W * m.in_size + m.inner * W
+            n += 2 * W * W
+            f = l.mlp
+            if f is not None:
+                n += 3 * W * f.ff * f.experts + 3 * W * f.shared_ff + W * f.routes
+        return n
+
+    def to_dict(self) -> dict:
+        return dataclasses.asdict(self)
+
+    @staticmethod
+    def from_dict(d: dict, name: str = "tifepel") -> "TifepelConfig":
+        layers = []
+        for e in d["layers"]:
+            m = e["mixer"]
+            if e["type"] == "attention":
+                qt = m.get("q_temp") or {}
+                spec = AttentionSpec(
+                    heads=int(m["heads"]), kv_heads=int(m["kv_heads"]), dim=int(m["dim"]), vdim=int(m["vdim"]),
+                    scale=float(m["scale"]), rot=None, out_gate=False, qk_norm_weight=False,
+                    q_temp_coef=float(qt.get("coef") or 0.0), q_temp_every=int(qt.get("every") or 0),
+                    bias_rows=-1 if m.get("bias_max") else 0, bias_max=float(m.get("bias_max") or 0.0))
+                if spec.heads % spec.kv_heads:
+                    raise ValueError("Tifepel: heads must be a multiple of kv_heads")
+            elif e["type"] == "mamba2":
+                spec = Mamba2Spec(heads=int(m["heads"]), vdim=int(m["vdim"]), state=int(m["state"]),
+                                  groups=int(m["groups"]), conv=int(m["conv"]),
+                                  norm_groups=int(m.get("norm_groups") or 1))
+                if spec.heads % spec.groups or spec.inner % spec.norm_groups:
+                    raise ValueError("Tifepel: heads must divide into groups and the inner width into norm groups")
+            else:
+                raise ValueError(f"Tifepel: unknown mixer type {e['type']!r}")
+            f = e.get("mlp")
+            mlp = None
+            if f is not None:
+                if f.get("kind", "moe") != "moe":
+                    raise ValueError(f"Tifepel: unknown feed-forward kind {f.get('kind')!r}")
+                r = f["router"]
+                mlp = MoeSpec(experts=int(r["experts"]), identity=int(r.get("identity") or 0), top=int(r["top"]),
+                              ff=int(f["expert"]["ff"]), shared_ff=int((f.get("shared") or {}).get("ff") or 0))
+            layers.append(LayerSpec(e["type"], spec, mlp))
+        bg = (d.get("embedding") or {}).get("bigram") or {}
+        lp = d.get("loop") or {}
+        return TifepelConfig(
+            name=name, vocab_size=int(d["vocab"]), hidden_size=int(d["width"]), layers=layers,
+            streams=int(d.get("streams") or 1), canon_taps=int((d.get("canon") or {}).get("taps") or 0),
+            bigram_buckets=int(bg.get("buckets") or 0), bigram_mul_prev=int(bg.get("mul_prev") or 0),
+            bigram_mul_cur=int(bg.get("mul_cur") or 0), loop_start=int(lp.get("start") or 0),
+            loop_stop=int(lp.get("stop") or 0), loop_times=int(lp.get("times") or 1),
+            norm_eps=float((d.get("norm") or {}).get("eps", 1e-6)), max_position=int(d.get("max_positions") or 2048))
+
+
+def tifepel_uniform(name: str, vocab: int, width: int, pattern: str, heads: int, kv_heads: int, dim: int, vdim: int,
+                    m_heads: int, m_vdim: int, state: int, groups: int, experts: int, identity: int, top: int, ff: int,
+                    shared_ff: int, bias_rows: int = 32, bias_max: float = 128.0, norm_groups: int = 1, conv: int = 4,
+                    **kw) -> TifepelConfig:
+    """A Tifepel configuration from a layer pattern ('a' attention, 'm' Mamba-2), all layers of a
+    kind sharing one geometry (presets, benchmarks)."""
+    layers = []
+    for ch in pattern:
+        if ch == "a":
+            mixer = AttentionSpec(heads, kv_heads, dim, vdim, dim ** -0.5, None, out_gate=False, qk_norm_weight=False,
+                                  q_temp_coef=0.25, q_temp_every=128, bias_rows=bias_rows, bias_max=bias_max)
+        else:
+            mixer = Mamba2Spec(m_heads, m_vdim, state, groups, conv, norm_groups)
+        layers.append(LayerSpec("attention" if ch == "a" else "mamba2", mixer,
+                                MoeSpec(experts, identity, top, ff, shared_ff) if ff else None))
+    return TifepelConfig(name=name, vocab_size=vocab, hidden_size=width, layers=layers, **kw)
+
+
+NATIVE_CONFIGS = {"bebovik": BebovikConfig.from_dict, "tifepel": TifepelConfig.from_dict}
 
 
 PRESETS: dict[str, ModelConfig] = {
@@ -324,6 +536,11 @@ PRESETS: dict[str, ModelConfig] = {
     "bebovik-tiny": bebovik_uniform("bebovik-tiny", 1024, 256, 3, 4, 2, 64, 64, 512, 48, rot_dims=16,
                                     embedding_scale=4.0, logit_scale=0.5, logit_softcap=30.0, max_position=4096,
                                     bos_token_id=1, eos_token_id=2),
+    # Tifepel test / smoke sizes (random weights): attention + Mamba-2 layers, the first two run twice
+    "tifepel-tiny": tifepel_uniform("tifepel-tiny", 512, 128, "amma", 4, 2, 32, 32, 4, 32, 32, 2, 6, 2, 2, 64, 64,
+                                    bias_rows=12, bias_max=40.0, norm_groups=2, streams=2, canon_taps=3,
+                                    bigram_buckets=251, bigram_mul_prev=31, bigram_mul_cur=7, loop_start=0,
+                                    loop_stop=2, loop_times=2, max_position=2048, bos_token_id=1, eos_token_id=2),
     "opt-125m": ModelConfig(name="opt-125m", arch="opt", vocab_size=50272, hidden_size=768,
                             intermediate_size=3072, num_layers=12, num_heads=12, num_kv_heads=12, head_dim=64,
                             max_position=2048, tie_embeddings=True, bos_token_id=2, eos_token_id=2),
@@ -353,7 +570,7 @@ def get_config(name_or_path: str) -> ModelConfig:
     if "@L" in name_or_path:
         base, n = name_or_path.rsplit("@L", 1)
         bc = get_config(base)
-        if isinstance(bc, BebovikConfig):
+        if isinstance(bc, (BebovikConfig, TifepelConfig)):
             return dataclasses.replace(bc, name=name_or_path, layers=bc.layers[: int(n)])
         return dataclasses.replace(bc, name=name_or_path, num_layers=int(n))
     key = ALIASES.get(name_or_path, name_or_path)

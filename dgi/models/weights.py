@@ -225,3 +225,77 @@ def load_bebovik_checkpoint(model, path: str) -> dict:
     out = {"tensors": n, "bytes": rd.bytes_read, "path": path}
     rd.close()
     return out
+
+
+def tifepel_bias_rows(cfg, path: str) -> None:
+    """Set every attention layer's ``bias_rows`` from the shape of its distance-bias table in the
+    checkpoint (the configuration file gives only the distance at which the buckets end)."""
+    rd = CheckpointReader(path)
+    for i, l in enumerate(cfg.layers):
+        if l.type == "attention" and l.mixer.bias_rows:
+            l.mixer.bias_rows = int(rd._h(f"l{i}.mix.rel").get_slice(f"l{i}.mix.rel").get_shape()[0])
+    rd.close()
+
+
+def load_tifepel_checkpoint(model, path: str) -> dict:
+    """Fill a ``TifepelModel`` from the design's safetensors layout: ``embed`` / ``bigram`` / ``pos`` /
+    ``head`` / ``final.norm`` and per layer i ``l<i>.norm{1,2}``, ``l<i>.canon{1,2}``, ``l<i>.rg{1,2}``
+    (+ ``.b``), ``l<i>.hc{1,2}.{in,out,mix}``, the mixer under ``l<i>.mix.`` (attention: q, k, v, rel, o;
+    Mamba-2: in, conv, conv.b, dt_bias, A_log, D, norm, o) and the feed-forward under ``l<i>.mlp.``
+    (router, correction, e<j>.{gate,up,down}, shared.{gate,up,down}).  q | k | v land in one fused
+    weight, every expert's gate | up in one stacked tensor; norm weights, convolution taps, stream
+    coefficients, the router and the scan's per-head constants stay fp32."""
+    rd = CheckpointReader(path)
+    n = 0
+
+    def put(dst, name):
+        nonlocal n
+        src = rd.read(name)
+        if src.dim() == dst.dim() and src.shape[0] < dst.shape[0] and src.shape[1:] == dst.shape[1:]:
+            dst = dst[: src.shape[0]]        # a table the engine made longer than the checkpoint's
+        _put(dst, src.reshape(dst.shape) if src.numel() == dst.numel() and src.dim() != dst.dim() else src)
+        n += 1
+
+    for i, L in enumerate(model.layers):
+        p = f"l{i}."
+        m, f = L.spec.mixer, L.spec.mlp
+        for q in ("1", "2") if f is not None else ("1",):
+            put(getattr(L, "norm" + q), p + "norm" + q)
+            if getattr(L, "canon" + q) is not None:
+                put(getattr(L, "canon" + q), p + "canon" + q)
+            put(getattr(L, "rg" + q), p + "rg" + q)
+            put(getattr(L, f"rg{q}_b"), f"{p}rg{q}.b")
+            for k in ("in", "out", "mix"):
+                put(getattr(L, f"hc{q}_{k}"), f"{p}hc{q}.{k}")
+        if L.spec.type == "attention":
+            r = 0
+            for key, rows in (("q", m.q_size), ("k", m.k_size), ("v", m.v_size)):
+                put(L.qkv[r:r + rows], p + "mix." + key)
+                r += rows
+            if L.rel is not None:
+                put(L.rel, p + "mix.rel")
+        else:
+            for dst, key in ((L.in_proj, "in"), (L.conv, "conv"), (L.conv_b, "conv.b"), (L.dt_bias, "dt_bias"),
+                             (L.a_log, "A_log"), (L.d_skip, "D"), (L.mnorm, "norm")):
+                put(dst, p + "mix." + key)
+        put(L.o, p + "mix.o")
+        if f is not None:
+            put(L.router, p + "mlp.router")
+            put(L.correction, p + "mlp.correction")
+            for e in range(f.experts):
+                put(L.gate_up[e, : f.ff], f"{p}mlp.e{e}.gate")
+                put(L.gate_up[e, f.ff:], f"{p}mlp.e{e}.up")
+                put(L.down[e], f"{p}mlp.e{e}.down")
+            if f.shared_ff:
+                put(L.shared_gate_up[: f.shared_ff], p + "mlp.shared.gate")
+                put(L.shared_gate_up[f.shared_ff:], p + "mlp.shared.up")
+                put(L.shared_down, p + "mlp.shared.down")
+    put(model.embed, "embed")
+    if model.bigram is not None:
+        put(model.bigram, "bigram")
+    put(model.pos, "pos")
+    put(model.head, "head")
+    put(model.final_norm, "final.norm")
+    out = {"tensors": n, "bytes": rd.bytes_read, "path": path}
+    rd.close()
+    return out

@@ -125,7 +125,8 @@ def _rot_pairs(x: torch.Tensor, cs: torch.Tensor) -> torch.Tensor:
     return torch.cat([r, x[..., rd:]], dim=-1)
 
 
-def qknorm_rope_cache_ref(qkv, positions, slots, qw, kw, eps, cos_sin, H, G, dk, dv, k_cache, v_cache) -> None:
+def qknorm_rope_cache_ref(qkv, positions, slots, qw, kw, eps, cos_sin, H, G, dk, dv, k_cache, v_cache,
+                          q_temp=None) -> None:
     T = qkv.shape[0]
     if T == 0:
         return
@@ -135,6 +136,9 @@ def qknorm_rope_cache_ref(qkv, positions, slots, qw, kw, eps, cos_sin, H, G, dk,
     v = qkv[:, (H + G) * dk:(H + G) * dk + G * dv].view(T, G, dv)
     q = q / torch.sqrt(q.pow(2).mean(-1, keepdim=True) + eps) * qw
     k = k / torch.sqrt(k.pow(2).mean(-1, keepdim=True) + eps) * kw
+    if q_temp is not None and q_temp[1] > 0:
+        steps = torch.div(positions.long() + 1, int(q_temp[1]), rounding_mode="floor")
+        q = q * (1.0 + float(q_temp[0]) * torch.log(steps.float() + 1.0))[:, None, None]
     if cos_sin is not None:
         cs = cos_sin[positions.long()]
         q, k = _rot_pairs(q, cs), _rot_pairs(k, cs)
@@ -147,22 +151,37 @@ def qknorm_rope_cache_ref(qkv, positions, slots, qw, kw, eps, cos_sin, H, G, dk,
 
 
 def qknorm_rope_cache(qkv, positions, slots, qw, kw, eps: float, cos_sin, H: int, G: int, dk: int, dv: int,
-                      k_cache, v_cache) -> None:
+                      k_cache, v_cache, q_temp=None) -> None:
     """Rows of ``qkv`` = [q: H*dk | k: G*dk | v: G*dv | ...]: per-head RMS norm (weights ``qw`` /
     ``kw`` [dk], eps inside the root) and interleaved rotary (``cos_sin`` [max_pos, rd], or None)
     of q in place and of k into ``k_cache`` [NB, G, bs, dk]; v into ``v_cache`` [NB, G, bs, dv]
-    at ``slots`` (-1: not written)."""
+    at ``slots`` (-1: not written).  ``q_temp`` = (coef, every): the normalised q of a row at
+    position p is also multiplied by 1 + coef * ln(floor((p + 1) / every) + 1)."""
+    qt = (float(q_temp[0]), int(q_temp[1])) if q_temp is not None else (0.0, 0)
     if _native(qkv):
-        _call("qknorm_rope_cache", qkv, positions, slots, qw, kw, float(eps), cos_sin, H, G, dk, dv, k_cache, v_cache)
+        _call("qknorm_rope_cache", qkv, positions, slots, qw, kw, float(eps), cos_sin, H, G, dk, dv, k_cache, v_cache,
+              qt[0], qt[1])
     else:
-        qknorm_rope_cache_ref(qkv, positions, slots, qw, kw, eps, cos_sin, H, G, dk, dv, k_cache, v_cache)
+        qknorm_rope_cache_ref(qkv, positions, slots, qw, kw, eps, cos_sin, H, G, dk, dv, k_cache, v_cache, qt)
 
 
 # ----------------------------------------------------------------------------
 # Row-wise masked attention
 # ----------------------------------------------------------------------------
 
-def masked_attn_rows_ref(q, k_cache, v_cache, block_tables, cu_seqlens, positions, H, G, scale, mask, gate=None):
+def distance_bias_table(rel: torch.Tensor, far: float) -> torch.Tensor:
+    """fp32 bias by distance [n, H] from a bucketed table ``rel`` [rows, H]
+    (``dgi.models.config.distance_bucket``): row d is the bias at distance d, the last row serves
+    every distance beyond it (the buckets end at ``far``)."""
+    from dgi.models.config import distance_bucket
+    rows = rel.shape[0]
+    n = max(int(-(-far // 1)), rows // 2) + 1
+    idx = torch.tensor([distance_bucket(d, rows, far) for d in range(n)], dtype=torch.long, device=rel.device)
+    return rel.float()[idx].contiguous()
+
+
+def masked_attn_rows_ref(q, k_cache, v_cache, block_tables, cu_seqlens, positions, H, G, scale, mask, gate=None,
+                         dist_bias=None):
     T = q.shape[0]
     bs, dk, dv = k_cache.shape[2], k_cache.shape[3], v_cache.shape[3]
     out = torch.zeros(T, H * dv, dtype=q.dtype, device=q.device)
@@ -183,6 +202,9 @@ def masked_attn_rows_ref(q, k_cache, v_cache, block_tables, cu_seqlens, position
         v = v_cache[blk, :, keys % bs].float()
         qt = q[t, : H * dk].float().view(G, H // G, dk)
         s = torch.einsum("ghd,ngd->ghn", qt, k) * scale
+        if dist_bias is not None:
+            d = (p - keys).clamp(max=dist_bias.shape[0] - 1)
+            s = s + dist_bias[d].t().reshape(G, H // G, -1)
         o = torch.einsum("ghn,ngd->ghd", torch.softmax(s, dim=-1), v).reshape(H * dv)
         if gate is not None:
             o = o * torch.sigmoid(gate[t, : H * dv].float())
@@ -191,18 +213,20 @@ def masked_attn_rows_ref(q, k_cache, v_cache, block_tables, cu_seqlens, position
 
 
 def masked_attn_rows(q, k_cache, v_cache, block_tables, cu_seqlens, positions, H: int, G: int, scale: float,
-                     mask: int = 0, gate=None, out=None) -> torch.Tensor:
+                     mask: int = 0, gate=None, out=None, dist_bias=None) -> torch.Tensor:
     """Softmax attention of each row of ``q`` (position ``positions[t]``) over keys
     [floor(p / mask) * mask, p] of its sequence (``mask`` 0: [0, p]) read from the paged cache;
     rows map to ``block_tables`` rows through ``cu_seqlens`` (None: row i <-> table row i).
-    ``gate``: the output is multiplied by sigmoid(gate) element by element."""
+    ``gate``: the output is multiplied by sigmoid(gate) element by element.  ``dist_bias``
+    [n, H] fp32: added to the scaled score of a key at distance d = p - j, row min(d, n - 1)."""
     if _native(q):
         if out is None:
             out = torch.empty(q.shape[0], H * v_cache.shape[3], dtype=q.dtype, device=q.device)
         _call("masked_attn_rows", out, q, k_cache, v_cache, block_tables, cu_seqlens, positions, H, G, float(scale),
-              int(mask), gate)
+              int(mask), gate, dist_bias)
         return out
-    r = masked_attn_rows_ref(q, k_cache, v_cache, block_tables, cu_seqlens, positions, H, G, scale, mask, gate)
+    r = masked_attn_rows_ref(q, k_cache, v_cache, block_tables, cu_seqlens, positions, H, G, scale, mask, gate,
+                             dist_bias)
     if out is not None:
         out.copy_(r)
         return out

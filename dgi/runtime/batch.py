@@ -34,6 +34,11 @@ class AttnMeta:
     pre_tiles: Optional[torch.Tensor] = None          # [n_tiles, 2] int32
     tree_mask: Optional[torch.Tensor] = None          # [Bp, 64] int64 ancestor bits (EAGLE verify)
     tree_n: int = 0
+    # per-sequence state (models with a StatePool): the step's sequences are its decode rows, then
+    # its prompt portions
+    row_seq: Optional[torch.Tensor] = None            # [T] int32 sequence index of every row
+    seq_row0: Optional[torch.Tensor] = None           # [n_seq + 1] int32 first row of every sequence
+    seq_slots: Optional[torch.Tensor] = None          # [n_seq] int32 state slot (0: the reserved slot)
     # rows whose hidden state feeds the LM head (None = all rows)
     logits_indices: Optional[torch.Tensor] = None
 

@@ -104,9 +104,10 @@ def sampling_rows(sampled: list, ahead=0):
 class ModelRunner:
     def __init__(self, model, pool, max_num_seqs: int = 256, max_model_len: int = 8192,
                  max_num_batched_tokens: int = 8192, use_graphs: bool = True,
-                 graph_buckets=DEFAULT_BUCKETS, decode_part_size: int = 256, num_cus: int = 256):
+                 graph_buckets=DEFAULT_BUCKETS, decode_part_size: int = 256, num_cus: int = 256, state_pool=None):
         self.model = model
         self.pool = pool
+        self.state_pool = state_pool
         self.device = pool.device
         self.bs = pool.block_size
         self.max_num_seqs = max_num_seqs
@@ -116,7 +117,7 @@ class ModelRunner:
         self.num_cus = num_cus
         self.step_id = 0
         if hasattr(model, "attach_cache"):
-            model.attach_cache(pool)
+            model.attach_cache(pool, state_pool) if state_pool is not None else model.attach_cache(pool)
         else:
             model.kv_cache = pool.kv
         self.is_cuda = self.device.type == "cuda"
@@ -147,13 +148,13 @@ class ModelRunner:
         self._spans = []
         self.span_total_ms = 0.0
         self.graphs = None
-        if use_graphs and self.is_cuda and model.has_head:
+        if use_graphs and self.is_cuda and model.has_head and getattr(model, "supports_graphs", True):
             self.graphs = GraphRunner(self, [b for b in graph_buckets if b <= max_num_seqs])
 
     # ------------------------------------------------------------------ metadata
     # header layout (int64): the host-side shape of one step, shipped along
     # the pipeline so every stage rebuilds the same AttnMeta
-    H_LEN, H_T, H_NDP, H_NPRE, H_NB, H_MAXW, H_SPLITS, H_PART, H_NTILES, H_NLOG, H_STEP, H_FILT = range(1, 13)
+    H_LEN, H_T, H_NDP, H_NPRE, H_NB, H_MAXW, H_SPLITS, H_PART, H_NTILES, H_NLOG, H_STEP, H_FILT, H_NSEQ = range(1, 14)
     HEADER_SIZE = 16
 
     def prebuild_decode(self, reqs: list, ahead: int = 1) -> dict:
@@ -240,6 +241,17 @@ class ModelRunner:
             temps, seeds, topk, topp, filt = sampling_rows(sampled, 0 if seed_ahead is None else seed_ahead)
         parts = [ids, pos, slots, dec_bt.ravel(), dec_ctx, pre_bt.ravel(), cu, pctx, tiles_np.ravel(), lidx,
                  temps, seeds, topk, topp]
+        nseq = 0
+        if self.state_pool is not None:
+            # sequences of the step (decode rows, then portions): row -> sequence, first rows, state slots
+            nseq = ndp + nb
+            lens = np.concatenate([np.ones(ndp, np.int32), np.diff(cu).astype(np.int32)])
+            row0 = np.zeros(nseq + 1, np.int32)
+            np.cumsum(lens, out=row0[1:])
+            sslot = np.zeros(nseq, np.int32)
+            sslot[:nd] = [r.state_slot for r in sb.decode]
+            sslot[ndp:] = [c.req.state_slot for c in chunks]
+            parts += [np.repeat(np.arange(nseq, dtype=np.int32), lens), row0, sslot]
         flat = np.concatenate(parts)
         max_ctx = int(dec_ctx.max()) if ndp else 1
         if self.is_cuda and ndp:
@@ -248,8 +260,8 @@ class ModelRunner:
             splits, part = 1, 1 << 20
         hdr = np.zeros(self.HEADER_SIZE, np.int64)
         hdr[[self.H_LEN, self.H_T, self.H_NDP, self.H_NPRE, self.H_NB, self.H_MAXW, self.H_SPLITS, self.H_PART,
-             self.H_NTILES, self.H_NLOG, self.H_STEP, self.H_FILT]] = [flat.size, T, ndp, npre, nb, maxw, splits,
-                                                                      part, len(tiles_np), nlog, self.step_id, int(filt)]
+             self.H_NTILES, self.H_NLOG, self.H_STEP, self.H_FILT, self.H_NSEQ]] = [
+                 flat.size, T, ndp, npre, nb, maxw, splits, part, len(tiles_np), nlog, self.step_id, int(filt), nseq]
         return flat, hdr, sampled
 
     def meta_from_device(self, dev: torch.Tensor, hdr):
@@ -257,20 +269,25 @@ class ModelRunner:
         h = [int(x) for x in hdr]
         T, ndp, npre, nb, maxw = h[self.H_T], h[self.H_NDP], h[self.H_NPRE], h[self.H_NB], h[self.H_MAXW]
         ntiles, nlog = h[self.H_NTILES], h[self.H_NLOG]
+        nseq = h[self.H_NSEQ]
         sizes = [T, T, T, ndp * maxw, ndp, nb * maxw, nb + 1, nb, ntiles * 2, nlog, nlog, nlog, nlog, nlog]
+        if nseq:
+            sizes += [T, nseq + 1, nseq]
         views = []
         o = 0
         for sz in sizes:
             views.append(dev[o: o + sz])
             o += sz
         (d_ids, d_pos, d_slots, d_dbt, d_dctx, d_pbt, d_cu, d_pctx, d_tiles, d_lidx, d_temps, d_seeds,
-         d_topk, d_topp) = views
+         d_topk, d_topp) = views[:14]
         meta = AttnMeta(
             positions=d_pos, slot_mapping=d_slots, num_decode=ndp,
             dec_block_tables=d_dbt.view(ndp, maxw), dec_context_lens=d_dctx,
             dec_max_splits=h[self.H_SPLITS], dec_part_size=h[self.H_PART], dec_workspace=self.dec_ws,
             num_prefill_tokens=npre, pre_block_tables=d_pbt.view(nb, maxw), pre_cu_seqlens=d_cu,
             pre_context_lens=d_pctx, pre_tiles=d_tiles.view(-1, 2), logits_indices=d_lidx)
+        if nseq:
+            meta.row_seq, meta.seq_row0, meta.seq_slots = views[14:17]
         samp = SamplingMeta(d_temps.view(torch.float32), d_seeds.long(),
                             d_topk.long() if h[self.H_FILT] else None,
                             d_topp.view(torch.float32) if h[self.H_FILT] else None)

@@ -126,6 +126,9 @@ class Scheduler:
         # running sequences admitted at most (None: max_num_seqs); the TPOT-SLO budget sets it
         # to what the engine sustains at the SLO (dgi.sched.slo.StepBudget.admission_cap)
         self.admit_cap: Optional[int] = None
+        # StatePool of a model that carries per-sequence state (recurrent mixers, convolution
+        # tails): a sequence gets a slot when it is admitted and returns it with its pages
+        self.state_pool = None
 
     # ------------------------------------------------------------------ queue
     def add(self, req: Request) -> None:
@@ -173,13 +176,16 @@ class Scheduler:
             req.radix_path = []
         self.pool.free(req.blocks)
         req.blocks = []
+        if req.state_slot:
+            self.state_pool.free(req.state_slot)
+            req.state_slot = 0
 
     def _preempt(self, victim: Request) -> None:
         self.running.remove(victim)
         n = victim.num_computed
         nb = (n + self.bs - 1) // self.bs
         tier = self.host_tier
-        if tier is not None and n > 0 and nb <= len(victim.blocks) and nb <= tier.num_free:
+        if tier is not None and self.state_pool is None and n > 0 and nb <= len(victim.blocks) and nb <= tier.num_free:
             # swap out: the computed pages go to pinned host memory, nothing is recomputed
             victim.swapped = (tier.spill(victim.blocks[:nb]), n, None)
             self._release(victim, cache=False)
@@ -345,6 +351,8 @@ class Scheduler:
                     break
                 self.waiting.popleft()
                 continue
+            if self.state_pool is not None and self.state_pool.num_free == 0:
+                break
             toks = req.all_tokens()
             target = req.prefill_target
             cached_blocks: list[int] = []
@@ -372,6 +380,8 @@ class Scheduler:
             req.num_computed = start
             req.num_cached = start
             req.status = Status.RUNNING
+            if self.state_pool is not None:
+                req.state_slot = self.state_pool.allocate()
             self.running.append(req)
             prefill.append(PrefillChunk(req, start, n, start + n == target))
             budget -= n
