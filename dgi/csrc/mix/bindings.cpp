@@ -19,11 +19,12 @@ int dgi_embed_dyt(const long long* ids, const void* table, int vocab, float scal
                   const float* b, float* res, int is_f32, int T, int W, hipStream_t s);
 int dgi_qknorm_rope_cache(void* qkv, int is_f32, int T, int stride, const int* positions, const int* slots,
                           const float* qw, const float* kw, float eps, const float* cos_sin, int rd, int H, int G,
-                          int dk, int dv, void* k_cache, void* v_cache, int block_size, hipStream_t s);
+                          int dk, int dv, void* k_cache, void* v_cache, int block_size, float qt_coef, int qt_every,
+                          hipStream_t s);
 int dgi_masked_attn_rows(const void* q, int q_stride, const void* k_cache, const void* v_cache, const int* block_tables,
                          int bt_stride, const int* cu_seqlens, int n_seqs, const int* positions, int rows, int H, int G,
                          int dk, int dv, int block_size, float scale, int mask, const void* gate, int gate_stride,
-                         void* out, int out_stride, int is_f32, hipStream_t s);
+                         void* out, int out_stride, int is_f32, const float* dist_bias, int n_dist, hipStream_t s);
 int dgi_paged_prefill_masked(const void* q, int q_stride, const void* k_cache, const void* v_cache,
                              const int* block_tables, int bt_stride, const int* cu_seqlens_q, const int* context_lens,
                              const int* tiles, int n_tiles, void* out, int out_stride, int nh, int nkv, int hd,
@@ -32,6 +33,32 @@ int dgi_glu_clamped(const void* gu, int gu_stride, void* out, int is_f32, int T,
                     hipStream_t s);
 int dgi_scale_softcap(const void* x, int x_stride, float* out, int is_f32, int T, int V, float scale, float cap,
                       hipStream_t s);
+int dgi_embed_streams(float* xs, int S, int T, int W, const int* ids, const int* positions, const int* row_seq,
+                      const int* seq_row0, const int* seq_slots, int n_seq, int* prev_tok, const void* embed, int vocab,
+                      const void* bigram, int buckets, long long mul_prev, long long mul_cur, const void* pos_table,
+                      int max_pos, int is_f32, hipStream_t s);
+int dgi_hc_mix_norm(float* xs, int S, int T, int W, const void* y, int y_stride, const void* gate, int gate_stride,
+                    const float* gate_b, const float* mixm, const float* outc, const float* in_next, const float* norm_w,
+                    float eps, float* h32, void* hd, int is_f32, hipStream_t s);
+int dgi_causal_conv(void* out, int out_f32, const void* x, int x_f32, int x_stride, int T, int C, int taps, const float* w,
+                    const float* bias, float* tail, const int* positions, const int* row_seq, const int* seq_row0,
+                    const int* seq_slots, int n_seq, int act, int residual, hipStream_t s);
+int dgi_ssm_scan(float* y, const float* xbc, int xbc_stride, const void* dt_raw, int dt_f32, int dt_stride,
+                 const float* dt_bias, const float* a_log, const float* d_skip, float* state, const int* positions,
+                 const int* seq_row0, const int* seq_slots, int n_seq, int heads, int dv, int N, int G, hipStream_t s);
+int dgi_gated_group_norm(void* out, int out_f32, const float* y, const void* z, int z_f32, int z_stride, const float* w,
+                         int T, int C, int groups, float eps, hipStream_t s);
+int dgi_moe_route(int* idx, float* wts, const float* logits, int l_stride, const float* corr, int T, int R, int top,
+                  hipStream_t s);
+int dgi_silu_mul(void* out, const void* gu, int gu_stride, int rows, int I, int is_f32, hipStream_t s);
+int dgi_moe_pair_gate_up(float* mid, const void* h, int h_stride, const int* idx, const void* gate_up, int T, int E,
+                         int top, int ff, int W, int is_f32, hipStream_t s);
+int dgi_moe_pair_down(void* out, const float* mid, const void* h, int h_stride, const int* idx, const float* wts,
+                      const void* down, const void* shared, int shared_stride, int T, int E, int top, int ff, int W,
+                      int is_f32, hipStream_t s);
+int dgi_moe_combine(void* out, const void* ys, const int* where, const void* h, int h_stride, const int* idx,
+                    const float* wts, const void* shared, int shared_stride, int T, int E, int top, int W, int is_f32,
+                    hipStream_t s);
 }
 
 namespace {
@@ -106,7 +133,7 @@ void embed_dyt(at::Tensor res, const at::Tensor& ids, const at::Tensor& table, d
 // qkv rows: [q: H*dk | k: G*dk | v: G*dv | ...]; k_cache [NB, G, bs, dk], v_cache [NB, G, bs, dv]
 void qknorm_rope_cache(at::Tensor qkv, const at::Tensor& positions, const at::Tensor& slots, const at::Tensor& qw,
                        const at::Tensor& kw, double eps, const c10::optional<at::Tensor>& cos_sin, int64_t H, int64_t G,
-                       int64_t dk, int64_t dv, at::Tensor k_cache, at::Tensor v_cache) {
+                       int64_t dk, int64_t dv, at::Tensor k_cache, at::Tensor v_cache, double qt_coef, int64_t qt_every) {
   const int f = act_kind(qkv, "qkv");
   check_rows(qkv, "qkv");
   check_i32(positions, "positions"); check_i32(slots, "slots");
@@ -128,7 +155,8 @@ void qknorm_rope_cache(at::Tensor qkv, const at::Tensor& positions, const at::Te
   }
   check_rc(dgi_qknorm_rope_cache(qkv.data_ptr(), f, T, (int)qkv.stride(0), positions.data_ptr<int>(), slots.data_ptr<int>(),
                                  qw.data_ptr<float>(), kw.data_ptr<float>(), (float)eps, cs, rd, (int)H, (int)G, (int)dk,
-                                 (int)dv, k_cache.data_ptr(), v_cache.data_ptr(), (int)k_cache.size(2), cur_stream()),
+                                 (int)dv, k_cache.data_ptr(), v_cache.data_ptr(), (int)k_cache.size(2), (float)qt_coef,
+                                 (int)qt_every, cur_stream()),
            "qknorm_rope_cache");
 }
 
@@ -137,7 +165,7 @@ void qknorm_rope_cache(at::Tensor qkv, const at::Tensor& positions, const at::Te
 void masked_attn_rows(at::Tensor out, const at::Tensor& q, const at::Tensor& k_cache, const at::Tensor& v_cache,
                       const at::Tensor& block_tables, const c10::optional<at::Tensor>& cu_seqlens,
                       const at::Tensor& positions, int64_t H, int64_t G, double scale, int64_t mask,
-                      const c10::optional<at::Tensor>& gate) {
+                      const c10::optional<at::Tensor>& gate, const c10::optional<at::Tensor>& dist_bias) {
   const int f = act_kind(q, "q");
   check_rows(q, "q"); check_rows(out, "out");
   TORCH_CHECK(act_kind(out, "out") == f && act_kind(k_cache, "k_cache") == f && act_kind(v_cache, "v_cache") == f);
@@ -165,10 +193,18 @@ void masked_attn_rows(at::Tensor out, const at::Tensor& q, const at::Tensor& k_c
     gp = gate->data_ptr();
     gs = (int)gate->stride(0);
   }
+  const float* db = nullptr;
+  int nd = 0;
+  if (dist_bias.has_value()) {
+    check_f32(*dist_bias, "dist_bias");
+    TORCH_CHECK(dist_bias->dim() == 2 && dist_bias->size(1) == H && dist_bias->size(0) >= 1, "dist_bias must be [n, H]");
+    db = dist_bias->data_ptr<float>();
+    nd = (int)dist_bias->size(0);
+  }
   check_rc(dgi_masked_attn_rows(q.data_ptr(), (int)q.stride(0), k_cache.data_ptr(), v_cache.data_ptr(),
                                 block_tables.data_ptr<int>(), (int)block_tables.stride(0), cu, n_seqs,
                                 positions.data_ptr<int>(), rows, (int)H, (int)G, dk, dv, (int)k_cache.size(2), (float)scale,
-                                (int)mask, gp, gs, out.data_ptr(), (int)out.stride(0), f, cur_stream()),
+                                (int)mask, gp, gs, out.data_ptr(), (int)out.stride(0), f, db, nd, cur_stream()),
            "masked_attn_rows");
 }
 
@@ -225,6 +261,212 @@ void scale_softcap(at::Tensor out, const at::Tensor& x, double scale, double cap
                              (float)scale, (float)cap, cur_stream()), "scale_softcap");
 }
 
+const int* i32p(const at::Tensor& t, const char* name, int64_t numel = -1) {
+  check_i32(t, name);
+  TORCH_CHECK(numel < 0 || t.numel() == numel, name, " has ", t.numel(), " elements, expected ", numel);
+  return t.data_ptr<int>();
+}
+const float* f32p(const c10::optional<at::Tensor>& t, const char* name, int64_t numel) {
+  if (!t.has_value()) return nullptr;
+  check_f32(*t, name, numel);
+  return t->data_ptr<float>();
+}
+
+// xs [S, T, W] fp32 <- embed[id] + bigram[hash(prev, id)] + pos_table[pos]; prev_tok [slots] int32 state
+void embed_streams(at::Tensor xs, const at::Tensor& ids, const at::Tensor& positions, const at::Tensor& row_seq,
+                   const at::Tensor& seq_row0, const at::Tensor& seq_slots, at::Tensor prev_tok, const at::Tensor& embed,
+                   const c10::optional<at::Tensor>& bigram, const c10::optional<at::Tensor>& pos_table, int64_t buckets,
+                   int64_t mul_prev, int64_t mul_cur) {
+  const int f = act_kind(embed, "embed");
+  check_f32(xs, "xs");
+  TORCH_CHECK(xs.dim() == 3 && embed.dim() == 2 && embed.is_contiguous());
+  const int S = (int)xs.size(0), T = (int)xs.size(1), W = (int)xs.size(2);
+  TORCH_CHECK(embed.size(1) == W);
+  const int n_seq = (int)seq_slots.numel();
+  check_i32(prev_tok, "prev_tok");
+  const void *bp = nullptr, *pp = nullptr;
+  int max_pos = 0;
+  if (bigram.has_value()) {
+    TORCH_CHECK(act_kind(*bigram, "bigram") == f && bigram->is_contiguous() && bigram->dim() == 2 && bigram->size(1) == W &&
+                bigram->size(0) == buckets + 1, "bigram must be [buckets + 1, W]");
+    bp = bigram->data_ptr();
+  }
+  if (pos_table.has_value()) {
+    TORCH_CHECK(act_kind(*pos_table, "pos_table") == f && pos_table->is_contiguous() && pos_table->dim() == 2 &&
+                pos_table->size(1) == W);
+    pp = pos_table->data_ptr();
+    max_pos = (int)pos_table->size(0);
+  }
+  check_rc(dgi_embed_streams(xs.data_ptr<float>(), S, T, W, i32p(ids, "ids", T), i32p(positions, "positions", T),
+                             i32p(row_seq, "row_seq", T), i32p(seq_row0, "seq_row0", n_seq + 1), i32p(seq_slots, "seq_slots"),
+                             n_seq, prev_tok.data_ptr<int>(), embed.data_ptr(), (int)embed.size(0), bp, (int)buckets,
+                             (long long)mul_prev, (long long)mul_cur, pp, max_pos, f, cur_stream()), "embed_streams");
+}
+
+void hc_mix_norm(at::Tensor xs, const c10::optional<at::Tensor>& y, const c10::optional<at::Tensor>& gate,
+                 const c10::optional<at::Tensor>& gate_b, const c10::optional<at::Tensor>& mixm,
+                 const c10::optional<at::Tensor>& outc, const c10::optional<at::Tensor>& in_next,
+                 const c10::optional<at::Tensor>& norm_w, double eps, c10::optional<at::Tensor> h32,
+                 c10::optional<at::Tensor> hd) {
+  check_f32(xs, "xs");
+  TORCH_CHECK(xs.dim() == 3);
+  const int S = (int)xs.size(0), T = (int)xs.size(1), W = (int)xs.size(2);
+  int f = hd.has_value() ? 0 : 1;
+  const void *yp = nullptr, *gp = nullptr;
+  int ys = 0, gs = 0;
+  if (y.has_value()) {
+    f = act_kind(*y, "y");
+    check_rows(*y, "y");
+    TORCH_CHECK(y->size(0) == T && y->size(1) == W && mixm.has_value() && outc.has_value(), "hc_mix_norm: y needs mix / out");
+    yp = y->data_ptr(); ys = (int)y->stride(0);
+    if (gate.has_value()) {
+      check_rows(*gate, "gate");
+      TORCH_CHECK(act_kind(*gate, "gate") == f && gate->size(0) == T && gate->size(1) == W && gate_b.has_value());
+      gp = gate->data_ptr(); gs = (int)gate->stride(0);
+    }
+  }
+  float* hp = nullptr;
+  void* hdp = nullptr;
+  if (in_next.has_value()) {
+    TORCH_CHECK(norm_w.has_value() && h32.has_value(), "hc_mix_norm: the read-out needs norm_w and h32");
+    check_f32(*h32, "h32", (int64_t)T * W);
+    hp = h32->data_ptr<float>();
+    if (hd.has_value()) {
+      TORCH_CHECK(f == 0 && hd->scalar_type() == at::kBFloat16 && hd->is_contiguous() && hd->numel() == (int64_t)T * W && hd->is_cuda(),
+                  "hc_mix_norm: hd is the bfloat16 copy of h for bfloat16 models");
+      hdp = hd->data_ptr();
+    }
+  }
+  check_rc(dgi_hc_mix_norm(xs.data_ptr<float>(), S, T, W, yp, ys, gp, gs, gp ? f32p(gate_b, "gate_b", W) : nullptr,
+                           yp ? f32p(mixm, "mix", (int64_t)S * S) : nullptr, yp ? f32p(outc, "out", S) : nullptr,
+                           f32p(in_next, "in_next", S), in_next.has_value() ? f32p(norm_w, "norm_w", W) : nullptr,
+                           (float)eps, hp, hdp, f, cur_stream()), "hc_mix_norm");
+}
+
+void causal_conv(at::Tensor out, const at::Tensor& x, const at::Tensor& w, const c10::optional<at::Tensor>& bias,
+                 const c10::optional<at::Tensor>& tail, const at::Tensor& positions, const at::Tensor& row_seq,
+                 const at::Tensor& seq_row0, const at::Tensor& seq_slots, int64_t act, bool residual) {
+  const int xf = act_kind(x, "x"), of = act_kind(out, "out");
+  check_rows(x, "x");
+  const int T = (int)x.size(0), C = (int)x.size(1);
+  TORCH_CHECK(out.is_contiguous() && out.dim() == 2 && out.size(0) == T && out.size(1) == C);
+  check_f32(w, "w");
+  TORCH_CHECK(w.dim() == 2 && w.size(0) == C, "w must be [C, taps]");
+  const int taps = (int)w.size(1);
+  const int n_seq = (int)seq_slots.numel();
+  float* tp = nullptr;
+  if (tail.has_value()) {
+    check_f32(*tail, "tail");
+    TORCH_CHECK(tail->dim() == 3 && tail->size(1) == taps - 1 && tail->size(2) == C, "tail must be [slots, taps - 1, C]");
+    tp = tail->data_ptr<float>();
+  }
+  check_rc(dgi_causal_conv(out.data_ptr(), of, x.data_ptr(), xf, (int)x.stride(0), T, C, taps, w.data_ptr<float>(),
+                           f32p(bias, "bias", C), tp, i32p(positions, "positions", T), i32p(row_seq, "row_seq", T),
+                           i32p(seq_row0, "seq_row0", n_seq + 1), i32p(seq_slots, "seq_slots"), n_seq, (int)act,
+                           residual ? 1 : 0, cur_stream()), "causal_conv");
+}
+
+void ssm_scan(at::Tensor y, const at::Tensor& xbc, const at::Tensor& dt_raw, const at::Tensor& dt_bias,
+              const at::Tensor& a_log, const at::Tensor& d_skip, at::Tensor state, const at::Tensor& positions,
+              const at::Tensor& seq_row0, const at::Tensor& seq_slots, int64_t heads, int64_t dv, int64_t N, int64_t G) {
+  check_f32(y, "y"); check_f32(xbc, "xbc"); check_f32(state, "state");
+  const int df = act_kind(dt_raw, "dt_raw");
+  check_rows(dt_raw, "dt_raw");
+  const int T = (int)xbc.size(0);
+  TORCH_CHECK(xbc.dim() == 2 && xbc.size(1) == heads * dv + 2 * G * N, "xbc must be [T, heads*dv + 2*G*N]");
+  TORCH_CHECK(y.numel() == (int64_t)T * heads * dv && dt_raw.size(0) == T && dt_raw.size(1) == heads);
+  TORCH_CHECK(state.dim() == 4 && state.size(1) == heads && state.size(2) == N && state.size(3) == dv, "state geometry");
+  check_f32(dt_bias, "dt_bias", heads); check_f32(a_log, "a_log", heads); check_f32(d_skip, "d_skip", heads);
+  const int n_seq = (int)seq_slots.numel();
+  check_rc(dgi_ssm_scan(y.data_ptr<float>(), xbc.data_ptr<float>(), (int)xbc.stride(0), dt_raw.data_ptr(), df,
+                        (int)dt_raw.stride(0), dt_bias.data_ptr<float>(), a_log.data_ptr<float>(), d_skip.data_ptr<float>(),
+                        state.data_ptr<float>(), i32p(positions, "positions", T), i32p(seq_row0, "seq_row0", n_seq + 1),
+                        i32p(seq_slots, "seq_slots"), n_seq, (int)heads, (int)dv, (int)N, (int)G, cur_stream()), "ssm_scan");
+}
+
+void gated_group_norm(at::Tensor out, const at::Tensor& y, const at::Tensor& z, const at::Tensor& w, int64_t groups,
+                      double eps) {
+  check_f32(y, "y");
+  const int zf = act_kind(z, "z"), of = act_kind(out, "out");
+  check_rows(z, "z");
+  TORCH_CHECK(y.dim() == 2 && out.is_contiguous() && out.sizes() == y.sizes() && z.size(0) == y.size(0) && z.size(1) == y.size(1));
+  check_f32(w, "w", y.size(1));
+  check_rc(dgi_gated_group_norm(out.data_ptr(), of, y.data_ptr<float>(), z.data_ptr(), zf, (int)z.stride(0),
+                                w.data_ptr<float>(), (int)y.size(0), (int)y.size(1), (int)groups, (float)eps, cur_stream()),
+           "gated_group_norm");
+}
+
+void moe_route(at::Tensor idx, at::Tensor wts, const at::Tensor& logits, const at::Tensor& corr) {
+  check_i32(idx, "idx"); check_f32(wts, "wts");
+  TORCH_CHECK(logits.is_cuda() && logits.scalar_type() == at::kFloat && logits.dim() == 2 && logits.stride(1) == 1);
+  const int T = (int)logits.size(0), R = (int)logits.size(1);
+  TORCH_CHECK(idx.dim() == 2 && idx.size(0) == T && wts.sizes() == idx.sizes());
+  check_f32(corr, "correction", R);
+  check_rc(dgi_moe_route(idx.data_ptr<int>(), wts.data_ptr<float>(), logits.data_ptr<float>(), (int)logits.stride(0),
+                         corr.data_ptr<float>(), T, R, (int)idx.size(1), cur_stream()), "moe_route");
+}
+
+void silu_mul(at::Tensor out, const at::Tensor& gu) {
+  const int f = act_kind(gu, "gu");
+  check_rows(gu, "gu");
+  TORCH_CHECK(act_kind(out, "out") == f && out.is_contiguous() && out.dim() == 2 && out.size(0) == gu.size(0) &&
+              2 * out.size(1) == gu.size(1));
+  check_rc(dgi_silu_mul(out.data_ptr(), gu.data_ptr(), (int)gu.stride(0), (int)gu.size(0), (int)out.size(1), f, cur_stream()),
+           "silu_mul");
+}
+
+// gate_up [E, 2 ff, W], down [E, W, ff] in h's dtype; idx / wts [T, top]
+void moe_pair_gate_up(at::Tensor mid, const at::Tensor& h, const at::Tensor& idx, const at::Tensor& gate_up) {
+  const int f = act_kind(h, "h");
+  check_rows(h, "h"); check_f32(mid, "mid"); check_i32(idx, "idx");
+  TORCH_CHECK(act_kind(gate_up, "gate_up") == f && gate_up.is_contiguous() && gate_up.dim() == 3 && gate_up.size(2) == h.size(1));
+  const int T = (int)h.size(0), W = (int)h.size(1), E = (int)gate_up.size(0), ff = (int)gate_up.size(1) / 2;
+  TORCH_CHECK(idx.dim() == 2 && idx.size(0) == T && mid.numel() == (int64_t)T * idx.size(1) * ff);
+  check_rc(dgi_moe_pair_gate_up(mid.data_ptr<float>(), h.data_ptr(), (int)h.stride(0), idx.data_ptr<int>(), gate_up.data_ptr(),
+                                T, E, (int)idx.size(1), ff, W, f, cur_stream()), "moe_pair_gate_up");
+}
+
+void moe_pair_down(at::Tensor out, const at::Tensor& mid, const at::Tensor& h, const at::Tensor& idx, const at::Tensor& wts,
+                   const at::Tensor& down, const c10::optional<at::Tensor>& shared) {
+  const int f = act_kind(h, "h");
+  check_rows(h, "h"); check_f32(mid, "mid"); check_i32(idx, "idx"); check_f32(wts, "wts");
+  TORCH_CHECK(act_kind(down, "down") == f && down.is_contiguous() && down.dim() == 3 && down.size(1) == h.size(1));
+  const int T = (int)h.size(0), W = (int)h.size(1), E = (int)down.size(0), ff = (int)down.size(2);
+  TORCH_CHECK(act_kind(out, "out") == f && out.is_contiguous() && out.size(0) == T && out.size(1) == W);
+  TORCH_CHECK(idx.dim() == 2 && idx.size(0) == T && wts.sizes() == idx.sizes() && mid.numel() == (int64_t)T * idx.size(1) * ff);
+  const void* sp = nullptr;
+  int ss = 0;
+  if (shared.has_value()) {
+    check_rows(*shared, "shared");
+    TORCH_CHECK(act_kind(*shared, "shared") == f && shared->size(0) == T && shared->size(1) == W);
+    sp = shared->data_ptr(); ss = (int)shared->stride(0);
+  }
+  check_rc(dgi_moe_pair_down(out.data_ptr(), mid.data_ptr<float>(), h.data_ptr(), (int)h.stride(0), idx.data_ptr<int>(),
+                             wts.data_ptr<float>(), down.data_ptr(), sp, ss, T, E, (int)idx.size(1), ff, W, f, cur_stream()),
+           "moe_pair_down");
+}
+
+void moe_combine(at::Tensor out, const at::Tensor& ys, const at::Tensor& where, const at::Tensor& h, const at::Tensor& idx,
+                 const at::Tensor& wts, const c10::optional<at::Tensor>& shared, int64_t E) {
+  const int f = act_kind(h, "h");
+  check_rows(h, "h"); check_i32(idx, "idx"); check_f32(wts, "wts"); check_i32(where, "where");
+  const int T = (int)h.size(0), W = (int)h.size(1);
+  TORCH_CHECK(act_kind(out, "out") == f && out.is_contiguous() && out.size(0) == T && out.size(1) == W);
+  TORCH_CHECK(act_kind(ys, "ys") == f && ys.is_contiguous() && ys.dim() == 2 && ys.size(1) == W);
+  TORCH_CHECK(idx.dim() == 2 && idx.size(0) == T && wts.sizes() == idx.sizes() && where.numel() == idx.numel() &&
+              ys.size(0) == idx.numel());
+  const void* sp = nullptr;
+  int ss = 0;
+  if (shared.has_value()) {
+    check_rows(*shared, "shared");
+    TORCH_CHECK(act_kind(*shared, "shared") == f && shared->size(0) == T && shared->size(1) == W);
+    sp = shared->data_ptr(); ss = (int)shared->stride(0);
+  }
+  check_rc(dgi_moe_combine(out.data_ptr(), ys.data_ptr(), where.data_ptr<int>(), h.data_ptr(), (int)h.stride(0),
+                           idx.data_ptr<int>(), wts.data_ptr<float>(), sp, ss, T, (int)E, (int)idx.size(1), W, f, cur_stream()),
+           "moe_combine");
+}
+
 }  // namespace
 
 TORCH_LIBRARY_FRAGMENT(dgi, m) {
@@ -233,14 +475,30 @@ TORCH_LIBRARY_FRAGMENT(dgi, m) {
         "Tensor? alpha2, Tensor? w2, Tensor? b2) -> ()");
   m.def("embed_dyt(Tensor(a!) res, Tensor ids, Tensor table, float scale, Tensor alpha, Tensor w, Tensor b) -> ()");
   m.def("qknorm_rope_cache(Tensor(a!) qkv, Tensor positions, Tensor slots, Tensor qw, Tensor kw, float eps, "
-        "Tensor? cos_sin, int H, int G, int dk, int dv, Tensor(b!) k_cache, Tensor(c!) v_cache) -> ()");
+        "Tensor? cos_sin, int H, int G, int dk, int dv, Tensor(b!) k_cache, Tensor(c!) v_cache, float qt_coef=0.0, "
+        "int qt_every=0) -> ()");
   m.def("masked_attn_rows(Tensor(a!) out, Tensor q, Tensor k_cache, Tensor v_cache, Tensor block_tables, "
-        "Tensor? cu_seqlens, Tensor positions, int H, int G, float scale, int mask, Tensor? gate) -> ()");
+        "Tensor? cu_seqlens, Tensor positions, int H, int G, float scale, int mask, Tensor? gate, "
+        "Tensor? dist_bias=None) -> ()");
   m.def("paged_prefill_masked(Tensor(a!) out, Tensor q, Tensor k_cache, Tensor v_cache, Tensor block_tables, "
         "Tensor cu_seqlens_q, Tensor context_lens, Tensor tiles, int nh, int nkv, float scale, int mask, "
         "Tensor? gate) -> ()");
   m.def("glu_clamped(Tensor(a!) out, Tensor gu, float limit, float alpha) -> ()");
   m.def("scale_softcap(Tensor(a!) out, Tensor x, float scale, float cap) -> ()");
+  m.def("embed_streams(Tensor(a!) xs, Tensor ids, Tensor positions, Tensor row_seq, Tensor seq_row0, Tensor seq_slots, "
+        "Tensor(b!) prev_tok, Tensor embed, Tensor? bigram, Tensor? pos_table, int buckets, int mul_prev, int mul_cur) -> ()");
+  m.def("hc_mix_norm(Tensor(a!) xs, Tensor? y, Tensor? gate, Tensor? gate_b, Tensor? mix, Tensor? out, Tensor? in_next, "
+        "Tensor? norm_w, float eps, Tensor(b!)? h32, Tensor(c!)? hd) -> ()");
+  m.def("causal_conv(Tensor(a!) out, Tensor x, Tensor w, Tensor? bias, Tensor(b!)? tail, Tensor positions, Tensor row_seq, "
+        "Tensor seq_row0, Tensor seq_slots, int act, bool residual) -> ()");
+  m.def("ssm_scan(Tensor(a!) y, Tensor xbc, Tensor dt_raw, Tensor dt_bias, Tensor a_log, Tensor d_skip, Tensor(b!) state, "
+        "Tensor positions, Tensor seq_row0, Tensor seq_slots, int heads, int dv, int N, int G) -> ()");
+  m.def("gated_group_norm(Tensor(a!) out, Tensor y, Tensor z, Tensor w, int groups, float eps) -> ()");
+  m.def("moe_route(Tensor(a!) idx, Tensor(b!) wts, Tensor logits, Tensor correction) -> ()");
+  m.def("silu_mul(Tensor(a!) out, Tensor gu) -> ()");
+  m.def("moe_pair_gate_up(Tensor(a!) mid, Tensor h, Tensor idx, Tensor gate_up) -> ()");
+  m.def("moe_pair_down(Tensor(a!) out, Tensor mid, Tensor h, Tensor idx, Tensor wts, Tensor down, Tensor? shared) -> ()");
+  m.def("moe_combine(Tensor(a!) out, Tensor ys, Tensor where, Tensor h, Tensor idx, Tensor wts, Tensor? shared, int E) -> ()");
 }
 
 TORCH_LIBRARY_IMPL(dgi, CUDA, m) {
@@ -252,4 +510,14 @@ TORCH_LIBRARY_IMPL(dgi, CUDA, m) {
   m.impl("paged_prefill_masked", &paged_prefill_masked);
   m.impl("glu_clamped", &glu_clamped);
   m.impl("scale_softcap", &scale_softcap);
+  m.impl("embed_streams", &embed_streams);
+  m.impl("hc_mix_norm", &hc_mix_norm);
+  m.impl("causal_conv", &causal_conv);
+  m.impl("ssm_scan", &ssm_scan);
+  m.impl("gated_group_norm", &gated_group_norm);
+  m.impl("moe_route", &moe_route);
+  m.impl("silu_mul", &silu_mul);
+  m.impl("moe_pair_gate_up", &moe_pair_gate_up);
+  m.impl("moe_pair_down", &moe_pair_down);
+  m.impl("moe_combine", &moe_combine);
 }

@@ -15,6 +15,8 @@
 // straight from the cache (this step's keys are written before it runs), so the result does
 // not depend on how the prompt was cut into steps or on what else is in the batch.
 // Scores, the online softmax and the output accumulation are fp32; exp is the accurate expf.
+// Optional distance bias: dist_bias[min(p - j, n_dist - 1)][head] (fp32, one row per distance, the
+// last row for everything farther) is added to the scaled score of key j before the softmax.
 // Optional epilogue: out *= sigmoid(gate) element by element (the mixer's output gate, read
 // from the same fused projection row as q).
 //
@@ -71,7 +73,8 @@ __global__ __launch_bounds__(64) void masked_attn_rows_kernel(
     const T* __restrict__ q, int q_stride, const T* __restrict__ k_cache, const T* __restrict__ v_cache,
     const int* __restrict__ block_tables, int bt_stride, const int* __restrict__ cu_seqlens, int n_seqs,
     const int* __restrict__ positions, int G, int dk, int dv, int bs, float scale, int mask,
-    const T* __restrict__ gate, int gate_stride, T* __restrict__ out, int out_stride) {
+    const T* __restrict__ gate, int gate_stride, T* __restrict__ out, int out_stride,
+    const float* __restrict__ dist_bias, int n_dist) {
   __shared__ float qs[MAXDK];
   __shared__ float ps[64];
   __shared__ long long vo[64];
@@ -112,6 +115,7 @@ __global__ __launch_bounds__(64) void masked_attn_rows_kernel(
       const int blk = bt[key / bs];
       const long long slot = ((long long)blk * G + kvh) * bs + (key % bs);
       s = dot_row(qs, k_cache + slot * dk, dk) * scale;
+      if (dist_bias) s += dist_bias[(size_t)min(pos - key, n_dist - 1) * H + head];
       vbase = slot * dv;
     }
     const float m_new = fmaxf(m_run, wave_max(s));     // lane 0's key k0 is always visible: finite
@@ -164,7 +168,8 @@ __global__ __launch_bounds__(64 * GNW) void masked_attn_group_kernel(
     const T* __restrict__ q, int q_stride, const T* __restrict__ k_cache, const T* __restrict__ v_cache,
     const int* __restrict__ block_tables, int bt_stride, const int* __restrict__ cu_seqlens, int n_seqs,
     const int* __restrict__ positions, int H, int dk, int dv, int bs, float scale, int mask,
-    const T* __restrict__ gate, int gate_stride, T* __restrict__ out, int out_stride) {
+    const T* __restrict__ gate, int gate_stride, T* __restrict__ out, int out_stride,
+    const float* __restrict__ dist_bias, int n_dist) {
   constexpr int E = 16 / sizeof(T);
   extern __shared__ __attribute__((aligned(16))) float smem[];
   const int row = blockIdx.x, kvh = blockIdx.y, G = gridDim.y;
@@ -241,7 +246,11 @@ __global__ __launch_bounds__(64 * GNW) void masked_attn_group_kernel(
 #pragma unroll
     for (int i = 0; i < R; ++i) {
       if (i < r) {
-        const float s = ok ? sc[i] * scale : -__builtin_inff();
+        float s = -__builtin_inff();
+        if (ok) {
+          s = sc[i] * scale;
+          if (dist_bias) s += dist_bias[(size_t)min(pos - key, n_dist - 1) * H + kvh * r + i];
+        }
         const float m_new = fmaxf(m[i], wave_max(s));       // key k0 (lane 0) is visible: finite
         const float p = ok ? expf(s - m_new) : 0.f;
         const float corr = expf(m[i] - m_new);
@@ -341,12 +350,12 @@ template <typename T, int R, int VP>
 int launch_group(const void* q, int q_stride, const void* k_cache, const void* v_cache, const int* block_tables,
                  int bt_stride, const int* cu_seqlens, int n_seqs, const int* positions, int rows, int H, int G, int dk,
                  int dv, int bs, float scale, int mask, const void* gate, int gate_stride, void* out, int out_stride,
-                 hipStream_t s) {
+                 const float* dist_bias, int n_dist, hipStream_t s) {
   const size_t lds = (size_t)(R * dk + GNW * R * 64 + GNW * 64 + 2 * GNW * R + GNW * R * dv) * 4;
   if (lds > 64 * 1024) return -1;
   masked_attn_group_kernel<T, R, VP><<<dim3(rows, G), 64 * GNW, lds, s>>>(
       (const T*)q, q_stride, (const T*)k_cache, (const T*)v_cache, block_tables, bt_stride, cu_seqlens, n_seqs,
-      positions, H, dk, dv, bs, scale, mask, (const T*)gate, gate_stride, (T*)out, out_stride);
+      positions, H, dk, dv, bs, scale, mask, (const T*)gate, gate_stride, (T*)out, out_stride, dist_bias, n_dist);
   return 0;
 }
 
@@ -354,10 +363,11 @@ template <typename T>
 int dispatch_group(int r, int vpn, const void* q, int q_stride, const void* k_cache, const void* v_cache,
                    const int* block_tables, int bt_stride, const int* cu_seqlens, int n_seqs, const int* positions,
                    int rows, int H, int G, int dk, int dv, int bs, float scale, int mask, const void* gate,
-                   int gate_stride, void* out, int out_stride, hipStream_t s) {
+                   int gate_stride, void* out, int out_stride, const float* dist_bias, int n_dist, hipStream_t s) {
 #define DGI_GRP(RV, VPV)                                                                                       \
   return launch_group<T, RV, VPV>(q, q_stride, k_cache, v_cache, block_tables, bt_stride, cu_seqlens, n_seqs, \
-                                  positions, rows, H, G, dk, dv, bs, scale, mask, gate, gate_stride, out, out_stride, s)
+                                  positions, rows, H, G, dk, dv, bs, scale, mask, gate, gate_stride, out, out_stride, dist_bias, \
+                                  n_dist, s)
   if (vpn == 1) {
     if (r == 1) DGI_GRP(1, 1);
     if (r == 2) DGI_GRP(2, 1);
@@ -379,11 +389,12 @@ extern "C" int dgi_masked_attn_rows(const void* q, int q_stride, const void* k_c
                                     const int* block_tables, int bt_stride, const int* cu_seqlens, int n_seqs,
                                     const int* positions, int rows, int H, int G, int dk, int dv, int block_size,
                                     float scale, int mask, const void* gate, int gate_stride, void* out,
-                                    int out_stride, int is_f32, hipStream_t s) {
+                                    int out_stride, int is_f32, const float* dist_bias, int n_dist, hipStream_t s) {
   if (rows == 0) return 0;
   if (G <= 0 || H % G) return -2;
   if (dk > MAXDK || dv > 64 * MAXC || dk <= 0 || dv <= 0) return -3;
   if (H > 65535 || mask < 0) return -4;
+  if (dist_bias && n_dist < 1) return -5;
   {
     // grouped kernel where the geometry allows (see masked_attn_group_kernel)
     const int E = is_f32 ? 4 : 8, r = H / G;
@@ -392,10 +403,10 @@ extern "C" int dgi_masked_attn_rows(const void* q, int q_stride, const void* k_c
     if (dk % E == 0 && dv % E == 0 && r <= 8 && vpn <= 2 && r * dv <= 1024 && aligned && G <= 65535) {
       const int rc = is_f32 ? dispatch_group<float>(r, vpn, q, q_stride, k_cache, v_cache, block_tables, bt_stride, cu_seqlens,
                                                     n_seqs, positions, rows, H, G, dk, dv, block_size, scale, mask, gate,
-                                                    gate_stride, out, out_stride, s)
+                                                    gate_stride, out, out_stride, dist_bias, n_dist, s)
                             : dispatch_group<uint16_t>(r, vpn, q, q_stride, k_cache, v_cache, block_tables, bt_stride,
                                                        cu_seqlens, n_seqs, positions, rows, H, G, dk, dv, block_size, scale,
-                                                       mask, gate, gate_stride, out, out_stride, s);
+                                                       mask, gate, gate_stride, out, out_stride, dist_bias, n_dist, s);
       if (rc == 0) {
         DGI_CHECK_LAUNCH();
         return 0;
@@ -406,12 +417,13 @@ extern "C" int dgi_masked_attn_rows(const void* q, int q_stride, const void* k_c
   if (is_f32)
     masked_attn_rows_kernel<float><<<grid, 64, 0, s>>>(
         (const float*)q, q_stride, (const float*)k_cache, (const float*)v_cache, block_tables, bt_stride, cu_seqlens,
-        n_seqs, positions, G, dk, dv, block_size, scale, mask, (const float*)gate, gate_stride, (float*)out, out_stride);
+        n_seqs, positions, G, dk, dv, block_size, scale, mask, (const float*)gate, gate_stride, (float*)out, out_stride,
+        dist_bias, n_dist);
   else
     masked_attn_rows_kernel<uint16_t><<<grid, 64, 0, s>>>(
         (const uint16_t*)q, q_stride, (const uint16_t*)k_cache, (const uint16_t*)v_cache, block_tables, bt_stride,
         cu_seqlens, n_seqs, positions, G, dk, dv, block_size, scale, mask, (const uint16_t*)gate, gate_stride,
-        (uint16_t*)out, out_stride);
+        (uint16_t*)out, out_stride, dist_bias, n_dist);
   DGI_CHECK_LAUNCH();
   return 0;
 }

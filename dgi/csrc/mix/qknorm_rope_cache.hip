@@ -8,7 +8,9 @@
 // rot() turns the interleaved pairs (2i, 2i+1) of the first rd dims by the row's position; the
 // other dims pass through.  cos_sin is the fp32 table [max_pos, rd] (rd/2 cos | rd/2 sin) that
 // rope_cache.hip reads too (frequency scaling is folded into the table); rd = 0: no rotation.
-// The norm, its weight and the rotation are computed in fp32 whatever the activation dtype.
+// Optional query temperature (qt_every > 0): a row at position p has its normalised q multiplied
+// by 1 + qt_coef * ln(floor((p + 1) / qt_every) + 1) — attention that sharpens as the context grows.
+// The norm, its weight, the temperature and the rotation are computed in fp32 whatever the activation dtype.
 //
 // Cache layout per layer: k [num_blocks, G, block_size, dk], v [num_blocks, G, block_size, dv].
 // One workgroup per token; a wave owns one head at a time (sum of squares by wave reduction),
@@ -48,9 +50,11 @@ template <typename T>
 __global__ __launch_bounds__(256) void qknorm_rope_cache_kernel(
     T* __restrict__ qkv, int stride, const int* __restrict__ positions, const int* __restrict__ slots,
     const float* __restrict__ qw, const float* __restrict__ kw, float eps, const float* __restrict__ cos_sin,
-    int rd, int H, int G, int dk, int dv, T* __restrict__ k_cache, T* __restrict__ v_cache, int block_size) {
+    int rd, int H, int G, int dk, int dv, T* __restrict__ k_cache, T* __restrict__ v_cache, int block_size,
+    float qt_coef, int qt_every) {
   const int t = blockIdx.x;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const float qtemp = qt_every > 0 ? 1.f + qt_coef * logf((float)((positions[t] + 1) / qt_every + 1)) : 1.f;
   T* row = qkv + (size_t)t * stride;
   const int slot = slots ? slots[t] : -1;
   const int blk = slot >= 0 ? slot / block_size : 0;
@@ -86,7 +90,7 @@ __global__ __launch_bounds__(256) void qknorm_rope_cache_kernel(
       ss += xv[j][0] * xv[j][0] + xv[j][1] * xv[j][1];
     }
     ss = wave_sum(ss);
-    const float r = 1.f / sqrtf(ss * inv_dk + eps);
+    const float r = 1.f / sqrtf(ss * inv_dk + eps) * (head < H ? qtemp : 1.f);
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const int e = 2 * (lane + 64 * j);
@@ -134,9 +138,11 @@ template <typename T, int MAXCH>
 __global__ __launch_bounds__(1024) void qknorm_rope_cache_vec_kernel(
     T* __restrict__ qkv, int stride, const int* __restrict__ positions, const int* __restrict__ slots,
     const float* __restrict__ qw, const float* __restrict__ kw, float eps, const float* __restrict__ cos_sin,
-    int rd, int H, int G, int dk, int dv, T* __restrict__ k_cache, T* __restrict__ v_cache, int block_size) {
+    int rd, int H, int G, int dk, int dv, T* __restrict__ k_cache, T* __restrict__ v_cache, int block_size,
+    float qt_coef, int qt_every) {
   constexpr int E = 16 / sizeof(T);
   const int t = blockIdx.x;
+  const float qtemp = qt_every > 0 ? 1.f + qt_coef * logf((float)((positions[t] + 1) / qt_every + 1)) : 1.f;
   const int grp = threadIdx.x >> 4, l = threadIdx.x & 15;
   T* row = qkv + (size_t)t * stride;
   const int slot = slots ? slots[t] : -1;
@@ -173,7 +179,7 @@ __global__ __launch_bounds__(1024) void qknorm_rope_cache_vec_kernel(
     }
 #pragma unroll
     for (int o = 8; o > 0; o >>= 1) ss += __shfl_xor(ss, o, 64);
-    const float r = 1.f / sqrtf(ss * inv_dk + eps);
+    const float r = 1.f / sqrtf(ss * inv_dk + eps) * (head < H ? qtemp : 1.f);
 #pragma unroll
     for (int j = 0; j < MAXCH; ++j) {
       const int c = l + 16 * j;
@@ -232,7 +238,7 @@ __global__ __launch_bounds__(1024) void qknorm_rope_cache_vec_kernel(
 extern "C" int dgi_qknorm_rope_cache(void* qkv, int is_f32, int T, int stride, const int* positions,
                                      const int* slots, const float* qw, const float* kw, float eps,
                                      const float* cos_sin, int rd, int H, int G, int dk, int dv, void* k_cache,
-                                     void* v_cache, int block_size, hipStream_t s) {
+                                     void* v_cache, int block_size, float qt_coef, int qt_every, hipStream_t s) {
   if (T == 0) return 0;
   if (rd < 0 || rd > dk || (rd & 1)) return -2;
   if (dk > 512) return -3;
@@ -248,21 +254,21 @@ extern "C" int dgi_qknorm_rope_cache(void* qkv, int is_f32, int T, int stride, c
     const dim3 vgrid(T, (H + G + hpb - 1) / hpb);
     if (is_f32)
       qknorm_rope_cache_vec_kernel<float, 4><<<vgrid, vthreads, 0, s>>>((float*)qkv, stride, positions, slots, qw, kw, eps, cos_sin,
-                                                               rd, H, G, dk, dv, (float*)k_cache, (float*)v_cache, block_size);
+                                                               rd, H, G, dk, dv, (float*)k_cache, (float*)v_cache, block_size, qt_coef, qt_every);
     else
       qknorm_rope_cache_vec_kernel<uint16_t, 4><<<vgrid, vthreads, 0, s>>>((uint16_t*)qkv, stride, positions, slots, qw, kw, eps,
                                                                   cos_sin, rd, H, G, dk, dv, (uint16_t*)k_cache,
-                                                                  (uint16_t*)v_cache, block_size);
+                                                                  (uint16_t*)v_cache, block_size, qt_coef, qt_every);
     DGI_CHECK_LAUNCH();
     return 0;
   }
   if (is_f32)
     qknorm_rope_cache_kernel<float><<<T, 256, 0, s>>>((float*)qkv, stride, positions, slots, qw, kw, eps, cos_sin,
-                                                      rd, H, G, dk, dv, (float*)k_cache, (float*)v_cache, block_size);
+                                                      rd, H, G, dk, dv, (float*)k_cache, (float*)v_cache, block_size, qt_coef, qt_every);
   else
     qknorm_rope_cache_kernel<uint16_t><<<T, 256, 0, s>>>((uint16_t*)qkv, stride, positions, slots, qw, kw, eps,
                                                          cos_sin, rd, H, G, dk, dv, (uint16_t*)k_cache,
-                                                         (uint16_t*)v_cache, block_size);
+                                                         (uint16_t*)v_cache, block_size, qt_coef, qt_every);
   DGI_CHECK_LAUNCH();
   return 0;
 }

@@ -39,7 +39,7 @@ __device__ __forceinline__ float block_sum(float v, float* red) {
 
 template <typename T>
 __global__ __launch_bounds__(256) void embed_streams_kernel(
-    float* __restrict__ xs, int S, int T, int W, const int* __restrict__ ids, const int* __restrict__ positions,
+    float* __restrict__ xs, int S, int NT, int W, const int* __restrict__ ids, const int* __restrict__ positions,
     const int* __restrict__ row_seq, const int* __restrict__ seq_row0, const int* __restrict__ seq_slots,
     const int* __restrict__ prev_tok, const T* __restrict__ embed, int vocab, const T* __restrict__ bigram,
     int buckets, long long mul_prev, long long mul_cur, const T* __restrict__ pos_table, int max_pos) {
@@ -65,7 +65,7 @@ __global__ __launch_bounds__(256) void embed_streams_kernel(
     float v = ldf<T>(e + w);
     if (b) v += ldf<T>(b + w);
     if (p) v += ldf<T>(p + w);
-    for (int s = 0; s < S; ++s) xs[((size_t)s * T + row) * W + w] = v;
+    for (int s = 0; s < S; ++s) xs[((size_t)s * NT + row) * W + w] = v;
   }
 }
 
@@ -79,7 +79,7 @@ __global__ void store_last_token_kernel(int* __restrict__ prev_tok, const int* _
 
 template <typename T>
 __global__ __launch_bounds__(256) void hc_mix_norm_kernel(
-    float* __restrict__ xs, int S, int T, int W, const T* __restrict__ y, int y_stride, const T* __restrict__ gate,
+    float* __restrict__ xs, int S, int NT, int W, const T* __restrict__ y, int y_stride, const T* __restrict__ gate,
     int gate_stride, const float* __restrict__ gate_b, const float* __restrict__ mixm, const float* __restrict__ outc,
     const float* __restrict__ in_next, const float* __restrict__ norm_w, float eps, float* __restrict__ h32,
     T* __restrict__ hd) {
@@ -97,7 +97,7 @@ __global__ __launch_bounds__(256) void hc_mix_norm_kernel(
   for (int w = threadIdx.x; w < W; w += blockDim.x) {
     float x[MAXS];
 #pragma unroll
-    for (int s = 0; s < MAXS; ++s) x[s] = s < S ? xs[((size_t)s * T + row) * W + w] : 0.f;
+    for (int s = 0; s < MAXS; ++s) x[s] = s < S ? xs[((size_t)s * NT + row) * W + w] : 0.f;
     if (y) {
       float yy = ldf<T>(y + (size_t)row * y_stride + w);
       if (gate) yy *= 1.f / (1.f + expf(-(ldf<T>(gate + (size_t)row * gate_stride + w) + gate_b[w])));
@@ -110,7 +110,7 @@ __global__ __launch_bounds__(256) void hc_mix_norm_kernel(
           for (int s = 0; s < MAXS; ++s)
             if (s < S) a += cm[s * S + t] * x[s];
           a += co[t] * yy;
-          xs[((size_t)t * T + row) * W + w] = a;
+          xs[((size_t)t * NT + row) * W + w] = a;
         }
         nx[t] = a;
       }

@@ -351,7 +351,7 @@ class TifepelModel:
 
     def embed_tokens(self, input_ids: torch.Tensor, meta: AttnMeta) -> torch.Tensor:
         c = self.cfg
-        return recur.embed_streams(input_ids.to(torch.int32), meta.positions, meta.seq_row0, meta.seq_slots,
+        return recur.embed_streams(input_ids.to(torch.int32), meta.positions, meta.row_seq, meta.seq_row0, meta.seq_slots,
                                    self.state["prev_tok"], self.embed, self.bigram, self.pos, c.bigram_buckets,
                                    c.bigram_mul_prev, c.bigram_mul_cur, c.streams)
 

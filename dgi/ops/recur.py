@@ -31,7 +31,7 @@ def _seqs(positions, seq_row0, seq_slots):
 # Embedding: token row + hashed bigram row + position row, copied into S streams
 # ----------------------------------------------------------------------------
 
-def embed_streams_ref(ids, positions, seq_row0, seq_slots, prev_tok, embed, bigram, pos_table, buckets, mul_prev,
+def embed_streams_ref(ids, positions, row_seq, seq_row0, seq_slots, prev_tok, embed, bigram, pos_table, buckets, mul_prev,
                       mul_cur, streams):
     T = ids.shape[0]
     x = embed[ids.long()].float()
@@ -51,7 +51,7 @@ def embed_streams_ref(ids, positions, seq_row0, seq_slots, prev_tok, embed, bigr
     return x.unsqueeze(0).repeat(streams, 1, 1).contiguous()
 
 
-def embed_streams(ids, positions, seq_row0, seq_slots, prev_tok, embed, bigram, pos_table, buckets: int,
+def embed_streams(ids, positions, row_seq, seq_row0, seq_slots, prev_tok, embed, bigram, pos_table, buckets: int,
                   mul_prev: int, mul_cur: int, streams: int) -> torch.Tensor:
     """fp32 streams [S, T, W], each embed[id] + bigram[(prev * mul_prev + id * mul_cur) mod buckets]
     + pos_table[position]; a sequence's first token takes bigram row ``buckets``.  The previous
@@ -60,10 +60,10 @@ def embed_streams(ids, positions, seq_row0, seq_slots, prev_tok, embed, bigram, 
     if _native(embed):
         T, W = ids.shape[0], embed.shape[1]
         xs = torch.empty(streams, T, W, dtype=torch.float32, device=embed.device)
-        _call("embed_streams", xs, ids, positions, seq_row0, seq_slots, prev_tok, embed, bigram, pos_table,
+        _call("embed_streams", xs, ids, positions, row_seq, seq_row0, seq_slots, prev_tok, embed, bigram, pos_table,
               int(buckets), int(mul_prev), int(mul_cur))
         return xs
-    return embed_streams_ref(ids, positions, seq_row0, seq_slots, prev_tok, embed, bigram, pos_table, buckets,
+    return embed_streams_ref(ids, positions, row_seq, seq_row0, seq_slots, prev_tok, embed, bigram, pos_table, buckets,
                              mul_prev, mul_cur, streams)
 
 
