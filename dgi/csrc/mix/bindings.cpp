@@ -50,7 +50,7 @@ int dgi_gated_group_norm(void* out, int out_f32, const float* y, const void* z, 
                          int T, int C, int groups, float eps, hipStream_t s);
 int dgi_moe_route(int* idx, float* wts, const float* logits, int l_stride, const float* corr, int T, int R, int top,
                   hipStream_t s);
-int dgi_silu_mul(void* out, const void* gu, int gu_stride, int rows, int I, int is_f32, hipStream_t s);
+int dgi_glu_silu(void* out, const void* gu, int gu_stride, int rows, int I, int is_f32, hipStream_t s);
 int dgi_moe_pair_gate_up(float* mid, const void* h, int h_stride, const int* idx, const void* gate_up, int T, int E,
                          int top, int ff, int W, int is_f32, hipStream_t s);
 int dgi_moe_pair_down(void* out, const float* mid, const void* h, int h_stride, const int* idx, const float* wts,
@@ -406,13 +406,13 @@ void moe_route(at::Tensor idx, at::Tensor wts, const at::Tensor& logits, const a
                          corr.data_ptr<float>(), T, R, (int)idx.size(1), cur_stream()), "moe_route");
 }
 
-void silu_mul(at::Tensor out, const at::Tensor& gu) {
+void glu_silu(at::Tensor out, const at::Tensor& gu) {
   const int f = act_kind(gu, "gu");
   check_rows(gu, "gu");
   TORCH_CHECK(act_kind(out, "out") == f && out.is_contiguous() && out.dim() == 2 && out.size(0) == gu.size(0) &&
               2 * out.size(1) == gu.size(1));
-  check_rc(dgi_silu_mul(out.data_ptr(), gu.data_ptr(), (int)gu.stride(0), (int)gu.size(0), (int)out.size(1), f, cur_stream()),
-           "silu_mul");
+  check_rc(dgi_glu_silu(out.data_ptr(), gu.data_ptr(), (int)gu.stride(0), (int)gu.size(0), (int)out.size(1), f, cur_stream()),
+           "glu_silu");
 }
 
 // gate_up [E, 2 ff, W], down [E, W, ff] in h's dtype; idx / wts [T, top]
@@ -495,7 +495,7 @@ TORCH_LIBRARY_FRAGMENT(dgi, m) {
         "Tensor positions, Tensor seq_row0, Tensor seq_slots, int heads, int dv, int N, int G) -> ()");
   m.def("gated_group_norm(Tensor(a!) out, Tensor y, Tensor z, Tensor w, int groups, float eps) -> ()");
   m.def("moe_route(Tensor(a!) idx, Tensor(b!) wts, Tensor logits, Tensor correction) -> ()");
-  m.def("silu_mul(Tensor(a!) out, Tensor gu) -> ()");
+  m.def("glu_silu(Tensor(a!) out, Tensor gu) -> ()");
   m.def("moe_pair_gate_up(Tensor(a!) mid, Tensor h, Tensor idx, Tensor gate_up) -> ()");
   m.def("moe_pair_down(Tensor(a!) out, Tensor mid, Tensor h, Tensor idx, Tensor wts, Tensor down, Tensor? shared) -> ()");
   m.def("moe_combine(Tensor(a!) out, Tensor ys, Tensor where, Tensor h, Tensor idx, Tensor wts, Tensor? shared, int E) -> ()");
@@ -516,7 +516,7 @@ TORCH_LIBRARY_IMPL(dgi, CUDA, m) {
   m.impl("ssm_scan", &ssm_scan);
   m.impl("gated_group_norm", &gated_group_norm);
   m.impl("moe_route", &moe_route);
-  m.impl("silu_mul", &silu_mul);
+  m.impl("glu_silu", &glu_silu);
   m.impl("moe_pair_gate_up", &moe_pair_gate_up);
   m.impl("moe_pair_down", &moe_pair_down);
   m.impl("moe_combine", &moe_combine);

@@ -179,7 +179,7 @@ extern "C" int dgi_moe_route(int* idx, float* wts, const float* logits, int l_st
   return 0;
 }
 
-extern "C" int dgi_silu_mul(void* out, const void* gu, int gu_stride, int rows, int I, int is_f32, hipStream_t s) {
+extern "C" int dgi_glu_silu(void* out, const void* gu, int gu_stride, int rows, int I, int is_f32, hipStream_t s) {
   if (rows == 0 || I == 0) return 0;
   const size_t n = (size_t)rows * I;
   const int blocks = (int)((n + 255) / 256 > 65535 ? 65535 : (n + 255) / 256);

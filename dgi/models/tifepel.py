@@ -71,7 +71,6 @@ class TifepelModel:
     """A Tifepel causal LM (all layers on one device)."""
 
     routes_gemms = False       # projections are plain vendor GEMMs: no start-up routing table
-    supports_graphs = False    # the step reads per-sequence state through host-built sequence tables
 
     def __init__(self, cfg: TifepelConfig, device: torch.device | str = "cpu", dtype=torch.bfloat16,
                  layer_start: int = 0, layer_end: Optional[int] = None, has_embed: Optional[bool] = None,

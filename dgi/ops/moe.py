@@ -38,7 +38,7 @@ def silu_mul(gu: torch.Tensor) -> torch.Tensor:
     """silu(g) * u over fused [gate | up] rows."""
     if _native(gu):
         out = torch.empty(gu.shape[0], gu.shape[1] // 2, dtype=gu.dtype, device=gu.device)
-        _call("silu_mul", out, gu)
+        _call("glu_silu", out, gu)
         return out
     return silu_mul_ref(gu)
 

@@ -413,17 +413,18 @@ class GraphRunner:
         dev = runner.device
         maxb = self.max_bucket
         maxw = runner.max_blocks
-        # one int32 staging image per replay: ids | pos | slots | ctx | temps | seeds | topk | topp
+        # one int32 staging image per replay: ids | pos | slots | ctx | temps | seeds | topk | topp | state slot
         # (b entries each) | block tables (b x maxw).  The pinned host copy lands in ``dev_in``
         # with ONE H2D copy and each bucket's graph reads its inputs straight out of it (round 3
         # copied nine device views into separate static tensors: nine copy launches per step)
-        self.NSEG = 8
+        self.NSEG = 9
         self.host_in2 = [torch.zeros(maxb * (self.NSEG + maxw), dtype=torch.int32).pin_memory() for _ in range(2)]
         self.host_out2 = [torch.zeros(maxb, dtype=torch.long).pin_memory() for _ in range(2)]
         self._flip = 0
         self.dev_in = torch.zeros(maxb * (self.NSEG + maxw), dtype=torch.int32, device=dev)
         self.out = torch.zeros(maxb, dtype=torch.long, device=dev)
         self.captured = False
+        self._rows = None
         # optional EAGLE-3 feature tap captured with the step: (layer ids, fuse fn) -> [b, H] per bucket
         self.features = None
         self.feats_out: dict = {}
@@ -449,17 +450,23 @@ class GraphRunner:
         S, d = self.NSEG, self.dev_in
         seg = d[: S * b].view(S, b)
         return {"ids": seg[0], "pos": seg[1], "slots": seg[2], "ctx": seg[3], "temps": seg[4].view(torch.float32),
-                "seeds": seg[5], "topk": seg[6], "topp": seg[7].view(torch.float32),
+                "seeds": seg[5], "topk": seg[6], "topp": seg[7].view(torch.float32), "sslot": seg[8],
                 "bt": d[S * b: S * b + b * self.r.max_blocks].view(b, self.r.max_blocks)}
 
     def _meta(self, b):
         r = self.r
         v = self.views(b)
         splits, part = (1, 1 << 20) if self._short else self.split_plan(b)
-        return AttnMeta(positions=v["pos"], slot_mapping=v["slots"], num_decode=b,
+        meta = AttnMeta(positions=v["pos"], slot_mapping=v["slots"], num_decode=b,
                         dec_block_tables=v["bt"], dec_context_lens=v["ctx"],
                         dec_max_splits=splits, dec_part_size=part, dec_workspace=r.dec_ws,
                         num_prefill_tokens=0, logits_indices=None)
+        if r.state_pool is not None:
+            # every row is a sequence of its own; padded rows use the reserved slot at position 0
+            if self._rows is None:
+                self._rows = torch.arange(self.max_bucket + 1, dtype=torch.int32, device=r.device)
+            meta.row_seq, meta.seq_row0, meta.seq_slots = self._rows[:b], self._rows[: b + 1], v["sslot"]
+        return meta
 
     def _body(self, b):
         m = self.r.model
@@ -542,6 +549,8 @@ class GraphRunner:
         tb, seeds[:n], topk[:n], pb, _f = sampling_rows(dec, ahead)
         temps[:n] = tb.view(np.float32)
         topp[:n] = pb.view(np.float32)
+        if r.state_pool is not None:
+            seg[8][:n] = [q.state_slot for q in dec]
         max_ctx = int(ctx[:n].max()) if n else 0
         k = S * b + b * maxw
         self.dev_in[:k].copy_(host_in[:k], non_blocking=True)

@@ -607,18 +607,22 @@ def test_checkpoint_layout_and_trace_runner(tmp_path):
 
 
 @pytest.mark.gpu
-def test_kernels_match_the_reference_ops_on_a_prompt_batch():
-    """bf16 on the GPU against the fp32 CPU reference ops through the same engine code: within
-    rounding over a batch of portions and decode rows."""
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_kernels_match_the_reference_ops_on_a_prompt_batch(dtype):
+    """The HIP kernels against the CPU reference ops through the same engine code, over a batch of
+    portions and decode rows: fp32 within rounding at every position; bf16 at the typical position
+    (one expert choice that flips on a close call moves a whole row, so rows are judged by their median)."""
     cfg = small_cfg()
-    cpu, gpu = engine(cfg, "cpu"), engine(cfg, "cuda", dtype=torch.bfloat16)
-    gpu.model.copy_from(cpu.model)
-    cpu.model.copy_from(gpu.model)                       # both hold the bf16-rounded weights
+    cpu, gpu = engine(cfg, "cpu", dtype=dtype), engine(cfg, "cuda", dtype=dtype)
+    cpu.model.copy_from(gpu.model)
     a, b = toks(50, 50), toks(33, 51)
     for eng in (cpu, gpu):
         eng.out = [eng.feed([("a", a[:40], list(range(40))), ("b", b[:2], [0, 1])]),
                    eng.feed([("a", a[40:41], [0]), ("b", b[2:], list(range(31)))]),
                    eng.feed([("a", a[41:], list(range(9)))], ["a", "b"])]
-    for x, y in zip(cpu.out, gpu.out):
-        for u, v in zip(x, y):
-            close(v, u, 0.3)
+    x = torch.cat([u for o in cpu.out for u in o], 0)
+    y = torch.cat([v for o in gpu.out for v in o], 0).cpu()
+    if dtype == torch.float32:
+        close(y, x, 3e-4)
+    else:
+        assert (y - x).abs().amax(1).median().item() < 0.1
