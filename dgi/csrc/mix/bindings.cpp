@@ -28,7 +28,8 @@ int dgi_masked_attn_rows(const void* q, int q_stride, const void* k_cache, const
 int dgi_paged_prefill_masked(const void* q, int q_stride, const void* k_cache, const void* v_cache,
                              const int* block_tables, int bt_stride, const int* cu_seqlens_q, const int* context_lens,
                              const int* tiles, int n_tiles, void* out, int out_stride, int nh, int nkv, int hd,
-                             int block_size, float scale, int mask, const void* gate, int gate_stride, hipStream_t s);
+                             int block_size, float scale, int mask, const void* gate, int gate_stride,
+                             const float* dist_bias, int n_dist, hipStream_t s);
 int dgi_glu_clamped(const void* gu, int gu_stride, void* out, int is_f32, int T, int I, float limit, float alpha,
                     hipStream_t s);
 int dgi_scale_softcap(const void* x, int x_stride, float* out, int is_f32, int T, int V, float scale, float cap,
@@ -51,11 +52,10 @@ int dgi_gated_group_norm(void* out, int out_f32, const float* y, const void* z, 
 int dgi_moe_route(int* idx, float* wts, const float* logits, int l_stride, const float* corr, int T, int R, int top,
                   hipStream_t s);
 int dgi_glu_silu(void* out, const void* gu, int gu_stride, int rows, int I, int is_f32, hipStream_t s);
-int dgi_moe_pair_gate_up(float* mid, const void* h, int h_stride, const int* idx, const void* gate_up, int T, int E,
-                         int top, int ff, int W, int is_f32, hipStream_t s);
-int dgi_moe_pair_down(void* out, const float* mid, const void* h, int h_stride, const int* idx, const float* wts,
-                      const void* down, const void* shared, int shared_stride, int T, int E, int top, int ff, int W,
-                      int is_f32, hipStream_t s);
+int dgi_moe_expert_gate_up(float* mid, const void* h, int h_stride, const int* idx, const void* gate_up, int T, int E,
+                           int top, int ff, int W, int is_f32, hipStream_t s);
+int dgi_moe_expert_down(void* ys, const float* mid, const int* idx, const void* down, int T, int E, int top, int ff, int W,
+                        int is_f32, hipStream_t s);
 int dgi_moe_combine(void* out, const void* ys, const int* where, const void* h, int h_stride, const int* idx,
                     const float* wts, const void* shared, int shared_stride, int T, int E, int top, int W, int is_f32,
                     hipStream_t s);
@@ -213,7 +213,7 @@ void masked_attn_rows(at::Tensor out, const at::Tensor& q, const at::Tensor& k_c
 void paged_prefill_masked(at::Tensor out, const at::Tensor& q, const at::Tensor& k_cache, const at::Tensor& v_cache,
                           const at::Tensor& block_tables, const at::Tensor& cu_seqlens_q, const at::Tensor& context_lens,
                           const at::Tensor& tiles, int64_t nh, int64_t nkv, double scale, int64_t mask,
-                          const c10::optional<at::Tensor>& gate) {
+                          const c10::optional<at::Tensor>& gate, const c10::optional<at::Tensor>& dist_bias) {
   TORCH_CHECK(act_kind(q, "q") == 0 && act_kind(out, "out") == 0 && act_kind(k_cache, "k_cache") == 0 &&
               act_kind(v_cache, "v_cache") == 0, "paged_prefill_masked: bfloat16 only");
   check_rows(q, "q"); check_rows(out, "out");
@@ -237,11 +237,19 @@ void paged_prefill_masked(at::Tensor out, const at::Tensor& q, const at::Tensor&
     gp = gate->data_ptr();
     gs = (int)gate->stride(0);
   }
+  const float* dbp = nullptr;
+  int ndist = 0;
+  if (dist_bias.has_value()) {
+    check_f32(*dist_bias, "dist_bias");
+    TORCH_CHECK(dist_bias->dim() == 2 && dist_bias->size(1) == nh && dist_bias->size(0) >= 1, "dist_bias must be [n, nh]");
+    dbp = dist_bias->data_ptr<float>();
+    ndist = (int)dist_bias->size(0);
+  }
   check_rc(dgi_paged_prefill_masked(q.data_ptr(), (int)q.stride(0), k_cache.data_ptr(), v_cache.data_ptr(),
                                     block_tables.data_ptr<int>(), (int)block_tables.stride(0), cu_seqlens_q.data_ptr<int>(),
                                     context_lens.data_ptr<int>(), tiles.data_ptr<int>(), (int)tiles.size(0), out.data_ptr(),
                                     (int)out.stride(0), (int)nh, (int)nkv, hd, (int)k_cache.size(2), (float)scale, (int)mask,
-                                    gp, gs, cur_stream()), "paged_prefill_masked");
+                                    gp, gs, dbp, ndist, cur_stream()), "paged_prefill_masked");
 }
 
 void glu_clamped(at::Tensor out, const at::Tensor& gu, double limit, double alpha) {
@@ -375,7 +383,7 @@ void ssm_scan(at::Tensor y, const at::Tensor& xbc, const at::Tensor& dt_raw, con
   const int T = (int)xbc.size(0);
   TORCH_CHECK(xbc.dim() == 2 && xbc.size(1) == heads * dv + 2 * G * N, "xbc must be [T, heads*dv + 2*G*N]");
   TORCH_CHECK(y.numel() == (int64_t)T * heads * dv && dt_raw.size(0) == T && dt_raw.size(1) == heads);
-  TORCH_CHECK(state.dim() == 4 && state.size(1) == heads && state.size(2) == N && state.size(3) == dv, "state geometry");
+  TORCH_CHECK(state.dim() == 4 && state.size(1) == heads && state.size(2) == dv && state.size(3) == N, "state must be [slots, heads, dv, N]");
   check_f32(dt_bias, "dt_bias", heads); check_f32(a_log, "a_log", heads); check_f32(d_skip, "d_skip", heads);
   const int n_seq = (int)seq_slots.numel();
   check_rc(dgi_ssm_scan(y.data_ptr<float>(), xbc.data_ptr<float>(), (int)xbc.stride(0), dt_raw.data_ptr(), df,
@@ -415,46 +423,42 @@ void glu_silu(at::Tensor out, const at::Tensor& gu) {
            "glu_silu");
 }
 
-// gate_up [E, 2 ff, W], down [E, W, ff] in h's dtype; idx / wts [T, top]
-void moe_pair_gate_up(at::Tensor mid, const at::Tensor& h, const at::Tensor& idx, const at::Tensor& gate_up) {
+// gate_up [E, 2 ff, W], down [E, W, ff] in h's dtype; idx [T, top]; mid [T * top, ff] fp32; ys [T * top, W]
+void moe_expert_gate_up(at::Tensor mid, const at::Tensor& h, const at::Tensor& idx, const at::Tensor& gate_up) {
   const int f = act_kind(h, "h");
   check_rows(h, "h"); check_f32(mid, "mid"); check_i32(idx, "idx");
   TORCH_CHECK(act_kind(gate_up, "gate_up") == f && gate_up.is_contiguous() && gate_up.dim() == 3 && gate_up.size(2) == h.size(1));
   const int T = (int)h.size(0), W = (int)h.size(1), E = (int)gate_up.size(0), ff = (int)gate_up.size(1) / 2;
   TORCH_CHECK(idx.dim() == 2 && idx.size(0) == T && mid.numel() == (int64_t)T * idx.size(1) * ff);
-  check_rc(dgi_moe_pair_gate_up(mid.data_ptr<float>(), h.data_ptr(), (int)h.stride(0), idx.data_ptr<int>(), gate_up.data_ptr(),
-                                T, E, (int)idx.size(1), ff, W, f, cur_stream()), "moe_pair_gate_up");
+  check_rc(dgi_moe_expert_gate_up(mid.data_ptr<float>(), h.data_ptr(), (int)h.stride(0), idx.data_ptr<int>(),
+                                  gate_up.data_ptr(), T, E, (int)idx.size(1), ff, W, f, cur_stream()), "moe_expert_gate_up");
 }
 
-void moe_pair_down(at::Tensor out, const at::Tensor& mid, const at::Tensor& h, const at::Tensor& idx, const at::Tensor& wts,
-                   const at::Tensor& down, const c10::optional<at::Tensor>& shared) {
-  const int f = act_kind(h, "h");
-  check_rows(h, "h"); check_f32(mid, "mid"); check_i32(idx, "idx"); check_f32(wts, "wts");
-  TORCH_CHECK(act_kind(down, "down") == f && down.is_contiguous() && down.dim() == 3 && down.size(1) == h.size(1));
-  const int T = (int)h.size(0), W = (int)h.size(1), E = (int)down.size(0), ff = (int)down.size(2);
-  TORCH_CHECK(act_kind(out, "out") == f && out.is_contiguous() && out.size(0) == T && out.size(1) == W);
-  TORCH_CHECK(idx.dim() == 2 && idx.size(0) == T && wts.sizes() == idx.sizes() && mid.numel() == (int64_t)T * idx.size(1) * ff);
-  const void* sp = nullptr;
-  int ss = 0;
-  if (shared.has_value()) {
-    check_rows(*shared, "shared");
-    TORCH_CHECK(act_kind(*shared, "shared") == f && shared->size(0) == T && shared->size(1) == W);
-    sp = shared->data_ptr(); ss = (int)shared->stride(0);
-  }
-  check_rc(dgi_moe_pair_down(out.data_ptr(), mid.data_ptr<float>(), h.data_ptr(), (int)h.stride(0), idx.data_ptr<int>(),
-                             wts.data_ptr<float>(), down.data_ptr(), sp, ss, T, E, (int)idx.size(1), ff, W, f, cur_stream()),
-           "moe_pair_down");
+void moe_expert_down(at::Tensor ys, const at::Tensor& mid, const at::Tensor& idx, const at::Tensor& down) {
+  const int f = act_kind(ys, "ys");
+  check_f32(mid, "mid"); check_i32(idx, "idx");
+  TORCH_CHECK(act_kind(down, "down") == f && down.is_contiguous() && down.dim() == 3);
+  const int E = (int)down.size(0), W = (int)down.size(1), ff = (int)down.size(2);
+  TORCH_CHECK(idx.dim() == 2 && ys.is_contiguous() && ys.dim() == 2 && ys.size(0) == idx.numel() && ys.size(1) == W &&
+              mid.numel() == idx.numel() * ff);
+  check_rc(dgi_moe_expert_down(ys.data_ptr(), mid.data_ptr<float>(), idx.data_ptr<int>(), down.data_ptr(), (int)idx.size(0), E,
+                               (int)idx.size(1), ff, W, f, cur_stream()), "moe_expert_down");
 }
 
-void moe_combine(at::Tensor out, const at::Tensor& ys, const at::Tensor& where, const at::Tensor& h, const at::Tensor& idx,
+void moe_combine(at::Tensor out, const at::Tensor& ys, const c10::optional<at::Tensor>& where, const at::Tensor& h, const at::Tensor& idx,
                  const at::Tensor& wts, const c10::optional<at::Tensor>& shared, int64_t E) {
   const int f = act_kind(h, "h");
-  check_rows(h, "h"); check_i32(idx, "idx"); check_f32(wts, "wts"); check_i32(where, "where");
+  check_rows(h, "h"); check_i32(idx, "idx"); check_f32(wts, "wts");
+  const int* wp = nullptr;
+  if (where.has_value()) {
+    check_i32(*where, "where");
+    TORCH_CHECK(where->numel() == idx.numel());
+    wp = where->data_ptr<int>();
+  }
   const int T = (int)h.size(0), W = (int)h.size(1);
   TORCH_CHECK(act_kind(out, "out") == f && out.is_contiguous() && out.size(0) == T && out.size(1) == W);
   TORCH_CHECK(act_kind(ys, "ys") == f && ys.is_contiguous() && ys.dim() == 2 && ys.size(1) == W);
-  TORCH_CHECK(idx.dim() == 2 && idx.size(0) == T && wts.sizes() == idx.sizes() && where.numel() == idx.numel() &&
-              ys.size(0) == idx.numel());
+  TORCH_CHECK(idx.dim() == 2 && idx.size(0) == T && wts.sizes() == idx.sizes() && ys.size(0) == idx.numel());
   const void* sp = nullptr;
   int ss = 0;
   if (shared.has_value()) {
@@ -462,7 +466,7 @@ void moe_combine(at::Tensor out, const at::Tensor& ys, const at::Tensor& where, 
     TORCH_CHECK(act_kind(*shared, "shared") == f && shared->size(0) == T && shared->size(1) == W);
     sp = shared->data_ptr(); ss = (int)shared->stride(0);
   }
-  check_rc(dgi_moe_combine(out.data_ptr(), ys.data_ptr(), where.data_ptr<int>(), h.data_ptr(), (int)h.stride(0),
+  check_rc(dgi_moe_combine(out.data_ptr(), ys.data_ptr(), wp, h.data_ptr(), (int)h.stride(0),
                            idx.data_ptr<int>(), wts.data_ptr<float>(), sp, ss, T, (int)E, (int)idx.size(1), W, f, cur_stream()),
            "moe_combine");
 }
@@ -482,7 +486,7 @@ TORCH_LIBRARY_FRAGMENT(dgi, m) {
         "Tensor? dist_bias=None) -> ()");
   m.def("paged_prefill_masked(Tensor(a!) out, Tensor q, Tensor k_cache, Tensor v_cache, Tensor block_tables, "
         "Tensor cu_seqlens_q, Tensor context_lens, Tensor tiles, int nh, int nkv, float scale, int mask, "
-        "Tensor? gate) -> ()");
+        "Tensor? gate, Tensor? dist_bias=None) -> ()");
   m.def("glu_clamped(Tensor(a!) out, Tensor gu, float limit, float alpha) -> ()");
   m.def("scale_softcap(Tensor(a!) out, Tensor x, float scale, float cap) -> ()");
   m.def("embed_streams(Tensor(a!) xs, Tensor ids, Tensor positions, Tensor row_seq, Tensor seq_row0, Tensor seq_slots, "
@@ -496,9 +500,9 @@ TORCH_LIBRARY_FRAGMENT(dgi, m) {
   m.def("gated_group_norm(Tensor(a!) out, Tensor y, Tensor z, Tensor w, int groups, float eps) -> ()");
   m.def("moe_route(Tensor(a!) idx, Tensor(b!) wts, Tensor logits, Tensor correction) -> ()");
   m.def("glu_silu(Tensor(a!) out, Tensor gu) -> ()");
-  m.def("moe_pair_gate_up(Tensor(a!) mid, Tensor h, Tensor idx, Tensor gate_up) -> ()");
-  m.def("moe_pair_down(Tensor(a!) out, Tensor mid, Tensor h, Tensor idx, Tensor wts, Tensor down, Tensor? shared) -> ()");
-  m.def("moe_combine(Tensor(a!) out, Tensor ys, Tensor where, Tensor h, Tensor idx, Tensor wts, Tensor? shared, int E) -> ()");
+  m.def("moe_expert_gate_up(Tensor(a!) mid, Tensor h, Tensor idx, Tensor gate_up) -> ()");
+  m.def("moe_expert_down(Tensor(a!) ys, Tensor mid, Tensor idx, Tensor down) -> ()");
+  m.def("moe_combine(Tensor(a!) out, Tensor ys, Tensor? where, Tensor h, Tensor idx, Tensor wts, Tensor? shared, int E) -> ()");
 }
 
 TORCH_LIBRARY_IMPL(dgi, CUDA, m) {
@@ -517,7 +521,7 @@ TORCH_LIBRARY_IMPL(dgi, CUDA, m) {
   m.impl("gated_group_norm", &gated_group_norm);
   m.impl("moe_route", &moe_route);
   m.impl("glu_silu", &glu_silu);
-  m.impl("moe_pair_gate_up", &moe_pair_gate_up);
-  m.impl("moe_pair_down", &moe_pair_down);
+  m.impl("moe_expert_gate_up", &moe_expert_gate_up);
+  m.impl("moe_expert_down", &moe_expert_down);
   m.impl("moe_combine", &moe_combine);
 }

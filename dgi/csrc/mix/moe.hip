@@ -4,14 +4,15 @@
 //   moe_route         one wave per token: s = softmax(logits) over all R routes (fp32), the `top` routes
 //                     with the largest s + correction (ties: lowest index), weights = s of those routes
 //   silu_mul          silu(g) * u over fused [gate | up] rows
-//   moe_pair_gate_up  grid (token * top + k, ff tiles): mid[pair][f] = silu(Wg[e] h)[f] * (Wu[e] h)[f],
-//                     straight from the stacked expert weights [E, 2 ff, W]; identity routes (e >= E) skip
-//   moe_pair_down     grid (token, W tiles): out[t][w] = sum_k wt_k * (Wd[e_k] mid_k)[w]  (identity: wt_k * h[t][w])
-//                     + shared[t][w]; the routes are added in their fixed order k = 0..top-1
-//   moe_combine       the same sum when the expert outputs sit in a buffer sorted by expert
-//                     (ys[where[pair]]), as the segment GEMMs of a large step leave them
+//   moe_expert_gate_up / moe_expert_down   small steps: grid (expert, output tile), each workgroup walks the
+//                     pairs that chose its expert straight from the stacked weights [E, 2 ff, W] / [E, W, ff]
+//                     (see below); identity routes (e >= E) belong to no workgroup
+//   moe_combine       out[t][w] = sum_k wt_k * ys[where[pair]][w]  (identity: wt_k * h[t][w]) + shared[t][w],
+//                     the routes added in their fixed order k = 0..top-1; `where` maps a pair to its row in
+//                     ys (null: the pair's own index), as the sorted segment GEMMs of a large step leave them
 //
 // Dot products run one output per wave with lanes striding the reduction dim, fp32 accumulation.
+#include <algorithm>
 #include "../common.h"
 
 using namespace dgi;
@@ -90,63 +91,117 @@ __global__ void silu_mul_kernel(T* __restrict__ out, const T* __restrict__ gu, i
   }
 }
 
-constexpr int OPW = 4;       // outputs per wave
+// ---------------------------------------------------------------------------------------------
+// Expert-major evaluation for small steps: a workgroup owns (expert e, a tile of outputs) and walks
+// the (token, route) pairs that chose e, PG at a time, so the expert's weight rows stream once per
+// group of PG pairs (once in all for a decode step with a handful of tokens per expert) instead of
+// once per pair.  The pairs of e are found by scanning idx and compacted into an LDS list (their
+// order there does not matter: every pair's result is independent).
+constexpr int CAP = 4096;    // pairs scanned per round
+constexpr int OPB = 32;      // outputs per workgroup (8 per wave)
 
-template <typename T>
-__global__ __launch_bounds__(256) void moe_pair_gate_up_kernel(
-    float* __restrict__ mid, const T* __restrict__ h, int h_stride, const int* __restrict__ idx,
-    const T* __restrict__ gate_up, int E, int top, int ff, int W) {
-  extern __shared__ float hs[];            // [W] the token's input
-  const int pair = blockIdx.x;
-  const int e = idx[pair];
-  if (e >= E || e < 0) return;             // identity route: nothing to project
-  const int t = pair / top;
-  for (int w = threadIdx.x; w < W; w += 256) hs[w] = ldf<T>(h + (size_t)t * h_stride + w);
+template <int PG>
+__device__ __forceinline__ int collect_pairs(const int* __restrict__ idx, int base, int P, int e, int* list, int* cnt) {
+  if (threadIdx.x == 0) *cnt = 0;
   __syncthreads();
+  const int hi = min(P, base + CAP);
+  for (int p = base + threadIdx.x; p < hi; p += blockDim.x)
+    if (idx[p] == e) list[atomicAdd(cnt, 1)] = p;
+  __syncthreads();
+  return *cnt;
+}
+
+// mid[pair][f] = silu(Wg[e][f] . h_t) * (Wu[e][f] . h_t)     gate_up [E, 2 ff, W]
+template <typename T, int PG>
+__global__ __launch_bounds__(256) void moe_expert_gate_up_kernel(
+    float* __restrict__ mid, const T* __restrict__ h, int h_stride, const int* __restrict__ idx,
+    const T* __restrict__ gate_up, int P, int top, int ff, int W) {
+  extern __shared__ __attribute__((aligned(16))) float sm[];
+  float* hs = sm;                                     // [PG][W]
+  int* list = reinterpret_cast<int*>(sm + (size_t)PG * W);   // [CAP]
+  __shared__ int cnt;
+  const int e = blockIdx.x;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const T* wg = gate_up + (size_t)e * 2 * ff * W;
-  for (int j = 0; j < OPW; ++j) {
-    const int f = (blockIdx.y * 4 + wave) * OPW + j;
-    if (f >= ff) break;
-    const T* gp = wg + (size_t)f * W;
-    const T* up = wg + (size_t)(ff + f) * W;
-    float ag = 0.f, au = 0.f;
-    for (int w = lane; w < W; w += 64) {
-      const float x = hs[w];
-      ag += ldf<T>(gp + w) * x;
-      au += ldf<T>(up + w) * x;
+  for (int base = 0; base < P; base += CAP) {
+    const int n = collect_pairs<PG>(idx, base, P, e, list, &cnt);
+    for (int g0 = 0; g0 < n; g0 += PG) {
+      const int np = min(PG, n - g0);
+      __syncthreads();                                // the previous group's rows are fully read
+      for (int i = threadIdx.x; i < PG * W; i += 256) {
+        const int p = i / W, w = i - p * W;
+        hs[i] = p < np ? ldf<T>(h + (size_t)(list[g0 + p] / top) * h_stride + w) : 0.f;
+      }
+      __syncthreads();
+      for (int j = 0; j < OPB / 4; ++j) {
+        const int f = blockIdx.y * OPB + wave * (OPB / 4) + j;
+        if (f >= ff) break;
+        const T* gp = wg + (size_t)f * W;
+        const T* up = wg + (size_t)(ff + f) * W;
+        float ag[PG], au[PG];
+#pragma unroll
+        for (int p = 0; p < PG; ++p) ag[p] = au[p] = 0.f;
+        for (int w = lane; w < W; w += 64) {
+          const float a = ldf<T>(gp + w), b = ldf<T>(up + w);
+#pragma unroll
+          for (int p = 0; p < PG; ++p) {
+            const float x = hs[p * W + w];
+            ag[p] += a * x;
+            au[p] += b * x;
+          }
+        }
+#pragma unroll
+        for (int p = 0; p < PG; ++p) {
+          const float sg = wave_sum(ag[p]), su = wave_sum(au[p]);
+          if (lane == 0 && p < np) mid[(size_t)list[g0 + p] * ff + f] = sg / (1.f + expf(-sg)) * su;
+        }
+      }
     }
-    ag = wave_sum(ag);
-    au = wave_sum(au);
-    if (lane == 0) mid[(size_t)pair * ff + f] = ag / (1.f + expf(-ag)) * au;
+    __syncthreads();                                  // list is rebuilt by the next round
   }
 }
 
-template <typename T>
-__global__ __launch_bounds__(256) void moe_pair_down_kernel(
-    T* __restrict__ out, const float* __restrict__ mid, const T* __restrict__ h, int h_stride,
-    const int* __restrict__ idx, const float* __restrict__ wts, const T* __restrict__ down, const T* __restrict__ shared,
-    int shared_stride, int E, int top, int ff, int W) {
-  const int t = blockIdx.x;
+// ys[pair][w] = Wd[e][w] . mid[pair]                           down [E, W, ff]
+template <typename T, int PG>
+__global__ __launch_bounds__(256) void moe_expert_down_kernel(
+    T* __restrict__ ys, const float* __restrict__ mid, const int* __restrict__ idx, const T* __restrict__ down, int P,
+    int ff, int W) {
+  extern __shared__ __attribute__((aligned(16))) float sm[];
+  float* ms = sm;                                     // [PG][ff]
+  int* list = reinterpret_cast<int*>(sm + (size_t)PG * ff);
+  __shared__ int cnt;
+  const int e = blockIdx.x;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-  for (int j = 0; j < OPW; ++j) {
-    const int w = (blockIdx.y * 4 + wave) * OPW + j;
-    if (w >= W) break;
-    float acc = shared ? ldf<T>(shared + (size_t)t * shared_stride + w) : 0.f;
-    for (int k = 0; k < top; ++k) {
-      const int e = idx[(size_t)t * top + k];
-      const float wt = wts[(size_t)t * top + k];
-      if (e >= E || e < 0) {
-        acc += wt * ldf<T>(h + (size_t)t * h_stride + w);
-      } else {
+  for (int base = 0; base < P; base += CAP) {
+    const int n = collect_pairs<PG>(idx, base, P, e, list, &cnt);
+    for (int g0 = 0; g0 < n; g0 += PG) {
+      const int np = min(PG, n - g0);
+      __syncthreads();
+      for (int i = threadIdx.x; i < PG * ff; i += 256) {
+        const int p = i / ff, f = i - p * ff;
+        ms[i] = p < np ? mid[(size_t)list[g0 + p] * ff + f] : 0.f;
+      }
+      __syncthreads();
+      for (int j = 0; j < OPB / 4; ++j) {
+        const int w = blockIdx.y * OPB + wave * (OPB / 4) + j;
+        if (w >= W) break;
         const T* dp = down + ((size_t)e * W + w) * ff;
-        const float* mp = mid + ((size_t)t * top + k) * ff;
-        float d = 0.f;
-        for (int f = lane; f < ff; f += 64) d += ldf<T>(dp + f) * mp[f];
-        acc += wt * wave_sum(d);
+        float acc[PG];
+#pragma unroll
+        for (int p = 0; p < PG; ++p) acc[p] = 0.f;
+        for (int f = lane; f < ff; f += 64) {
+          const float a = ldf<T>(dp + f);
+#pragma unroll
+          for (int p = 0; p < PG; ++p) acc[p] += a * ms[p * ff + f];
+        }
+#pragma unroll
+        for (int p = 0; p < PG; ++p) {
+          const float sd = wave_sum(acc[p]);
+          if (lane == 0 && p < np) stf<T>(ys + (size_t)list[g0 + p] * W + w, sd);
+        }
       }
     }
-    if (lane == 0) stf<T>(out + (size_t)t * W + w, acc);
+    __syncthreads();
   }
 }
 
@@ -163,7 +218,7 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(
     const int e = idx[(size_t)t * top + k];
     const float wt = wts[(size_t)t * top + k];
     if (e >= E || e < 0) acc += wt * ldf<T>(h + (size_t)t * h_stride + w);
-    else acc += wt * ldf<T>(ys + (size_t)where[(size_t)t * top + k] * W + w);
+    else acc += wt * ldf<T>(ys + (size_t)(where ? where[(size_t)t * top + k] : t * top + k) * W + w);
   }
   stf<T>(out + (size_t)t * W + w, acc);
 }
@@ -189,35 +244,43 @@ extern "C" int dgi_glu_silu(void* out, const void* gu, int gu_stride, int rows, 
   return 0;
 }
 
-extern "C" int dgi_moe_pair_gate_up(float* mid, const void* h, int h_stride, const int* idx, const void* gate_up,
-                                    int T, int E, int top, int ff, int W, int is_f32, hipStream_t s) {
-  if (T == 0) return 0;
-  if (W > 16384) return -2;
-  const dim3 grid(T * top, (ff + 4 * OPW - 1) / (4 * OPW));
+// pairs per group by LDS budget (PG rows of `row_len` floats + the pair list within 64 KiB)
+static int pick_pg(int row_len) {
+  const int room = (64 * 1024 - CAP * 4) / 4;
+  return row_len * 8 <= room ? 8 : (row_len * 4 <= room ? 4 : (row_len * 2 <= room ? 2 : (row_len <= room ? 1 : 0)));
+}
+
+extern "C" int dgi_moe_expert_gate_up(float* mid, const void* h, int h_stride, const int* idx, const void* gate_up,
+                                      int T, int E, int top, int ff, int W, int is_f32, hipStream_t s) {
+  if (T == 0 || E == 0) return 0;
+  const int pg = pick_pg(W);
+  if (!pg) return -2;
+  const dim3 grid(E, (ff + OPB - 1) / OPB);
   if (grid.y > 65535) return -3;
-  if (is_f32)
-    moe_pair_gate_up_kernel<float><<<grid, 256, (size_t)W * 4, s>>>(mid, (const float*)h, h_stride, idx,
-                                                                    (const float*)gate_up, E, top, ff, W);
-  else
-    moe_pair_gate_up_kernel<uint16_t><<<grid, 256, (size_t)W * 4, s>>>(mid, (const uint16_t*)h, h_stride, idx,
-                                                                       (const uint16_t*)gate_up, E, top, ff, W);
+  const size_t lds = ((size_t)pg * W + CAP) * 4;
+#define DGI_GU(TT_, PG_)                                                                                   \
+  moe_expert_gate_up_kernel<TT_, PG_><<<grid, 256, lds, s>>>(mid, (const TT_*)h, h_stride, idx, (const TT_*)gate_up, \
+                                                            T * top, top, ff, W)
+  if (is_f32) { if (pg == 8) DGI_GU(float, 8); else if (pg == 4) DGI_GU(float, 4); else if (pg == 2) DGI_GU(float, 2); else DGI_GU(float, 1); }
+  else { if (pg == 8) DGI_GU(uint16_t, 8); else if (pg == 4) DGI_GU(uint16_t, 4); else if (pg == 2) DGI_GU(uint16_t, 2); else DGI_GU(uint16_t, 1); }
+#undef DGI_GU
   DGI_CHECK_LAUNCH();
   return 0;
 }
 
-extern "C" int dgi_moe_pair_down(void* out, const float* mid, const void* h, int h_stride, const int* idx,
-                                 const float* wts, const void* down, const void* shared, int shared_stride, int T,
-                                 int E, int top, int ff, int W, int is_f32, hipStream_t s) {
-  if (T == 0) return 0;
-  const dim3 grid(T, (W + 4 * OPW - 1) / (4 * OPW));
+extern "C" int dgi_moe_expert_down(void* ys, const float* mid, const int* idx, const void* down, int T, int E, int top,
+                                   int ff, int W, int is_f32, hipStream_t s) {
+  if (T == 0 || E == 0) return 0;
+  const int pg = pick_pg(ff);
+  if (!pg) return -2;
+  const dim3 grid(E, (W + OPB - 1) / OPB);
   if (grid.y > 65535) return -3;
-  if (is_f32)
-    moe_pair_down_kernel<float><<<grid, 256, 0, s>>>((float*)out, mid, (const float*)h, h_stride, idx, wts,
-                                                     (const float*)down, (const float*)shared, shared_stride, E, top, ff, W);
-  else
-    moe_pair_down_kernel<uint16_t><<<grid, 256, 0, s>>>((uint16_t*)out, mid, (const uint16_t*)h, h_stride, idx, wts,
-                                                        (const uint16_t*)down, (const uint16_t*)shared, shared_stride, E,
-                                                        top, ff, W);
+  const size_t lds = ((size_t)pg * ff + CAP) * 4;
+#define DGI_DN(TT_, PG_) \
+  moe_expert_down_kernel<TT_, PG_><<<grid, 256, lds, s>>>((TT_*)ys, mid, idx, (const TT_*)down, T * top, ff, W)
+  if (is_f32) { if (pg == 8) DGI_DN(float, 8); else if (pg == 4) DGI_DN(float, 4); else if (pg == 2) DGI_DN(float, 2); else DGI_DN(float, 1); }
+  else { if (pg == 8) DGI_DN(uint16_t, 8); else if (pg == 4) DGI_DN(uint16_t, 4); else if (pg == 2) DGI_DN(uint16_t, 2); else DGI_DN(uint16_t, 1); }
+#undef DGI_DN
   DGI_CHECK_LAUNCH();
   return 0;
 }

@@ -7,13 +7,18 @@
 //     S  <- a * S + dt * B_t x_t^T                          S: [N, dv] fp32
 //     y_t = S^T C_t + d_skip[h] * x_t
 //
-// S starts as state[slot][h] (zero when the portion starts at position 0) and goes back there after
+// S starts as state[slot][h] (stored transposed, [dv][N]; zero when the portion starts at position 0) and goes back there after
 // the last row; decode rows (one token) and prompt portions run the same code, so the result does
 // not depend on how a prompt was cut.  x | B | C come as one fp32 row (the convolution's output).
 //
 // Work split: a workgroup owns (sequence, head, 16 value columns); thread (column v, n-lane l) keeps
-// S[n][v] for n = l + 16 i in registers, so the y reduction over n is four shuffles inside a 16-lane
-// group.  Everything is fp32 (softplus in its overflow-free form max(z, 0) + log1p(exp(-|z|))).
+// S[n][v] for n = 4 l + 64 q + j in registers, so the y reduction over n is four shuffles inside a
+// 16-lane group.  The serial loop over tokens never waits for global memory: B, C, x and the step
+// sizes of 16 tokens are staged in LDS (the next tile's loads are in flight, in registers, while the
+// current one is consumed; softplus and the decay are computed once per token while staging), and a
+// token costs two 16-byte LDS reads per four state values.  The state is stored value-major,
+// [slot][head][v][n], so a thread's values are contiguous.  Everything is fp32 (softplus in its
+// overflow-free form max(z, 0) + log1p(exp(-|z|))).
 //
 // gated_group_norm: g = y * silu(z), each of `groups` equal parts of a row divided by its own root
 // mean square (eps inside the root), times w.
@@ -32,16 +37,29 @@ template <> __device__ __forceinline__ void stf<uint16_t>(uint16_t* p, float v) 
 
 constexpr int COLS = 16;     // value columns per workgroup
 constexpr int NL = 16;       // n-lanes per column
+constexpr int TT = 16;       // tokens per staged tile
 
-template <typename TD, int NPT>
+// NQ: float4 groups of state per thread (N <= 64 * NQ); thread (column v, n-lane l) owns
+// n = 4 l + 64 q + j, j < 4.  LDS tile: B [TT][NP], C [TT][NP] (NP = 64 NQ, zero beyond N), x [TT][COLS],
+// dt [TT], decay [TT].
+template <typename TD, int NQ>
 __global__ __launch_bounds__(COLS * NL) void ssm_scan_kernel(
     float* __restrict__ y, const float* __restrict__ xbc, int xbc_stride, const TD* __restrict__ dt_raw, int dt_stride,
     const float* __restrict__ dt_bias, const float* __restrict__ a_log, const float* __restrict__ d_skip,
     float* __restrict__ state, const int* __restrict__ positions, const int* __restrict__ seq_row0,
     const int* __restrict__ seq_slots, int heads, int dv, int N, int G) {
+  constexpr int NP = 64 * NQ;
+  constexpr int PB = (TT * NP) / (COLS * NL);          // B (and C) values a thread stages per tile
+  extern __shared__ __attribute__((aligned(16))) float sm[];
+  float* sB = sm;
+  float* sC = sB + TT * NP;
+  float* sX = sC + TT * NP;
+  float* sDt = sX + TT * COLS;
+  float* sDa = sDt + TT;
   const int seq = blockIdx.x, h = blockIdx.y;
-  const int l = threadIdx.x & (NL - 1);
-  const int v = blockIdx.z * COLS + (threadIdx.x >> 4);
+  const int tid = threadIdx.x;
+  const int l = tid & (NL - 1), col = tid >> 4;
+  const int v = blockIdx.z * COLS + col;
   const int r0 = seq_row0[seq], r1 = seq_row0[seq + 1];
   if (r1 <= r0) return;
   const bool vok = v < dv;
@@ -49,42 +67,80 @@ __global__ __launch_bounds__(COLS * NL) void ssm_scan_kernel(
   const int inner = heads * dv;
   const float* bp = xbc + inner + (size_t)g * N;
   const float* cp = bp + (size_t)G * N;
-  float* sp = state + (((size_t)seq_slots[seq] * heads + h) * N) * dv + v;
-  float S[NPT];
+  float* sp = state + (((size_t)seq_slots[seq] * heads + h) * dv + v) * N;     // state [slot][head][v][n]
   const bool fresh = positions[r0] == 0;
+  float S[NQ][4];
 #pragma unroll
-  for (int i = 0; i < NPT; ++i) {
-    const int n = l + NL * i;
-    S[i] = (!fresh && vok && n < N) ? sp[(size_t)n * dv] : 0.f;
-  }
-  const float na = -expf(a_log[h]), bias = dt_bias[h], dsk = d_skip[h];
-  for (int t = r0; t < r1; ++t) {
-    const float z = ldf<TD>(dt_raw + (size_t)t * dt_stride + h) + bias;
-    const float dt = fmaxf(z, 0.f) + log1pf(expf(-fabsf(z)));
-    const float a = expf(na * dt);
-    const float* row = xbc + (size_t)t * xbc_stride;
-    const float xv = vok ? row[(size_t)h * dv + v] : 0.f;
-    const float dx = dt * xv;
-    float acc = 0.f;
+  for (int q = 0; q < NQ; ++q)
 #pragma unroll
-    for (int i = 0; i < NPT; ++i) {
-      const int n = l + NL * i;
-      if (n < N) {
-        const float bn = bp[(size_t)t * xbc_stride + n], cn = cp[(size_t)t * xbc_stride + n];
-        S[i] = a * S[i] + bn * dx;
-        acc += S[i] * cn;
-      }
+    for (int j = 0; j < 4; ++j) {
+      const int n = 4 * l + 64 * q + j;
+      S[q][j] = (!fresh && vok && n < N) ? sp[n] : 0.f;
     }
+  const float na = -expf(a_log[h]), bias = dt_bias[h], dsk = d_skip[h];
+
+  float rb[PB], rc[PB], rx = 0.f, rdt = 0.f;
+  auto prefetch = [&](int t0) {
 #pragma unroll
-    for (int o = NL / 2; o > 0; o >>= 1) acc += __shfl_xor(acc, o, 64);
-    if (l == 0 && vok) y[(size_t)t * inner + (size_t)h * dv + v] = acc + dsk * xv;
+    for (int i = 0; i < PB; ++i) {
+      const int idx = tid + i * (COLS * NL);
+      const int tok = idx / NP, n = idx - tok * NP;
+      const bool ok = t0 + tok < r1 && n < N;
+      rb[i] = ok ? bp[(size_t)(t0 + tok) * xbc_stride + n] : 0.f;
+      rc[i] = ok ? cp[(size_t)(t0 + tok) * xbc_stride + n] : 0.f;
+    }
+    {
+      const int tok = tid / COLS, c = tid - tok * COLS;            // TT * COLS == blockDim
+      const int vv = blockIdx.z * COLS + c;
+      rx = (t0 + tok < r1 && vv < dv) ? xbc[(size_t)(t0 + tok) * xbc_stride + (size_t)h * dv + vv] : 0.f;
+    }
+    if (tid < TT) rdt = t0 + tid < r1 ? ldf<TD>(dt_raw + (size_t)(t0 + tid) * dt_stride + h) : 0.f;
+  };
+  prefetch(r0);
+  for (int t0 = r0; t0 < r1; t0 += TT) {
+    __syncthreads();                                     // the previous tile is fully consumed
+#pragma unroll
+    for (int i = 0; i < PB; ++i) {
+      sB[tid + i * (COLS * NL)] = rb[i];
+      sC[tid + i * (COLS * NL)] = rc[i];
+    }
+    sX[tid] = rx;
+    if (tid < TT) {
+      const float z = rdt + bias;
+      const float dt = fmaxf(z, 0.f) + log1pf(expf(-fabsf(z)));
+      sDt[tid] = dt;
+      sDa[tid] = expf(na * dt);
+    }
+    __syncthreads();
+    if (t0 + TT < r1) prefetch(t0 + TT);                 // in flight while this tile is consumed
+    const int cnt = min(TT, r1 - t0);
+    for (int k = 0; k < cnt; ++k) {
+      const float a = sDa[k], xv = sX[k * COLS + col];
+      const float dx = sDt[k] * xv;
+      float acc = 0.f;
+#pragma unroll
+      for (int q = 0; q < NQ; ++q) {
+        const float4 b4 = *reinterpret_cast<const float4*>(sB + k * NP + 4 * l + 64 * q);
+        const float4 c4 = *reinterpret_cast<const float4*>(sC + k * NP + 4 * l + 64 * q);
+        S[q][0] = a * S[q][0] + b4.x * dx;
+        S[q][1] = a * S[q][1] + b4.y * dx;
+        S[q][2] = a * S[q][2] + b4.z * dx;
+        S[q][3] = a * S[q][3] + b4.w * dx;
+        acc += S[q][0] * c4.x + S[q][1] * c4.y + S[q][2] * c4.z + S[q][3] * c4.w;
+      }
+#pragma unroll
+      for (int o = NL / 2; o > 0; o >>= 1) acc += __shfl_xor(acc, o, 64);
+      if (l == 0 && vok) y[(size_t)(t0 + k) * inner + (size_t)h * dv + v] = acc + dsk * xv;
+    }
   }
   if (vok) {
 #pragma unroll
-    for (int i = 0; i < NPT; ++i) {
-      const int n = l + NL * i;
-      if (n < N) sp[(size_t)n * dv] = S[i];
-    }
+    for (int q = 0; q < NQ; ++q)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int n = 4 * l + 64 * q + j;
+        if (n < N) sp[n] = S[q][j];
+      }
   }
 }
 
@@ -122,17 +178,18 @@ extern "C" int dgi_ssm_scan(float* y, const float* xbc, int xbc_stride, const vo
                             int dv, int N, int G, hipStream_t s) {
   if (n_seq == 0) return 0;
   if (G <= 0 || heads % G) return -2;
-  if (N > NL * 16 || N <= 0 || dv <= 0) return -3;
+  if (N > 256 || N <= 0 || dv <= 0) return -3;
   const dim3 grid(n_seq, heads, (dv + COLS - 1) / COLS);
   if (heads > 65535 || grid.z > 65535) return -4;
-#define DGI_SCAN(TD, NPT)                                                                                            \
-  ssm_scan_kernel<TD, NPT><<<grid, COLS * NL, 0, s>>>(y, xbc, xbc_stride, (const TD*)dt_raw, dt_stride, dt_bias, a_log, \
-                                                      d_skip, state, positions, seq_row0, seq_slots, heads, dv, N, G)
-  const int npt = (N + NL - 1) / NL;
+#define DGI_SCAN(TD, NQ)                                                                                                \
+  ssm_scan_kernel<TD, NQ><<<grid, COLS * NL, (size_t)(2 * TT * 64 * NQ + TT * COLS + 2 * TT) * 4, s>>>(                 \
+      y, xbc, xbc_stride, (const TD*)dt_raw, dt_stride, dt_bias, a_log, d_skip, state, positions, seq_row0, seq_slots, \
+      heads, dv, N, G)
+  const int nq = (N + 63) / 64;
   if (dt_f32) {
-    if (npt <= 4) DGI_SCAN(float, 4); else if (npt <= 8) DGI_SCAN(float, 8); else DGI_SCAN(float, 16);
+    if (nq <= 1) DGI_SCAN(float, 1); else if (nq <= 2) DGI_SCAN(float, 2); else DGI_SCAN(float, 4);
   } else {
-    if (npt <= 4) DGI_SCAN(uint16_t, 4); else if (npt <= 8) DGI_SCAN(uint16_t, 8); else DGI_SCAN(uint16_t, 16);
+    if (nq <= 1) DGI_SCAN(uint16_t, 1); else if (nq <= 2) DGI_SCAN(uint16_t, 2); else DGI_SCAN(uint16_t, 4);
   }
 #undef DGI_SCAN
   DGI_CHECK_LAUNCH();

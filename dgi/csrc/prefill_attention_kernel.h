@@ -8,6 +8,8 @@
 //     tile is "interior" (no per-element mask) only when it lies inside the block of the
 //     wave's last row;
 //   * an output gate: out *= sigmoid(gate) element by element in the epilogue (fp32).
+// BIAS adds a learned distance bias to the scores before the mask: dist_bias[min(p - j, n_dist - 1)][head]
+// (fp32, natural score units; the kernel works in raw q.k units, hence inv_scale = 1 / scale).
 #pragma once
 #include "common.h"
 
@@ -42,14 +44,15 @@ constexpr int KT = 64;  // keys per tile
 // global loads are issued, then tile i is consumed — one barrier per 64 keys instead of
 // two, and a wave's LDS write no longer waits for every other wave before its MFMAs
 // (round 5: 24 % MFMA busy with DB = 0, profiles/r5_pmc/).
-template <int HD, int NW, int DB, bool MASKED = false>
+template <int HD, int NW, int DB, bool MASKED = false, bool BIAS = false>
 __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void prefill_attn_kernel(
     const uint16_t* __restrict__ q, int q_stride, const uint16_t* __restrict__ k_cache,
     const uint16_t* __restrict__ v_cache, const int* __restrict__ block_tables, int bt_stride,
     const int* __restrict__ cu_seqlens_q, const int* __restrict__ context_lens,
     const int* __restrict__ tiles, uint16_t* __restrict__ out, int out_stride, int nh, int nkv,
     int bs_log2, float scale_log2, const unsigned long long* __restrict__ tree_mask, int tree_n,
-    int mask = 0, const uint16_t* __restrict__ gate = nullptr, int gate_stride = 0) {
+    int mask = 0, const uint16_t* __restrict__ gate = nullptr, int gate_stride = 0,
+    const float* __restrict__ dist_bias = nullptr, int n_dist = 0, float inv_scale = 0.f) {
   __shared__ __attribute__((aligned(16))) uint16_t lds[(DB ? 2 : 1) * 2 * KT * HD];
 
   const int b = tiles[2 * blockIdx.x];
@@ -232,6 +235,26 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void prefill_attn_kernel(
       for (int s = 0; s < NS; ++s) {
         const u32x4 a = *reinterpret_cast<const u32x4*>(ks + k_off<HD>(32 * kb + lr, 2 * s + hh));
         sc[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16x8(a), as_bf16x8(qf[s]), sc[kb], 0, 0, 0);
+      }
+    }
+    if constexpr (BIAS) {
+      // distance bias in raw score units (bias / scale): one table row per distance, the last row for
+      // everything farther — a tile wholly beyond it for every row of the wave adds one constant
+      if (wave_first_pos - (kb0 + KT - 1) >= n_dist - 1) {
+        const float bl = dist_bias[(size_t)(n_dist - 1) * nh + head] * inv_scale;
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) sc[kb][r] += bl;
+      } else {
+        const int keyb = kb0 + 4 * hh;
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            const int d = my_pos - (keyb + 32 * kb + (r & 3) + 8 * (r >> 2));
+            sc[kb][r] += dist_bias[(size_t)min(max(d, 0), n_dist - 1) * nh + head] * inv_scale;
+          }
       }
     }
     // ---- online softmax; lane owns query lr, keys kb0 + 32kb + (r&3) + 8(r>>2) + 4hh.

@@ -27,7 +27,8 @@ Per layer run the step executes (rows: decode rows first, then packed prompt por
     gate GEMM              R h                                 (bias and sigmoid live in the next hc_mix_norm)
     causal_conv (HIP)      c = h + conv(h), tail in the sequence's state slot
     attention:  q|k|v GEMM -> qknorm_rope_cache (HIP: unit RMS, q temperature, paged K/V write)
-                -> masked_attn_rows (HIP, distance bias) -> o GEMM
+                -> masked_attn_rows (HIP, distance bias; prompt rows of bf16 64 / 128-dim heads: the MFMA
+                   flash kernel with the same bias) -> o GEMM
     mamba2:     in GEMM -> causal_conv (HIP, bias + SiLU, fp32 out) -> ssm_scan (HIP, fp32 state in the slot)
                 -> gated_group_norm (HIP) -> o GEMM
     moe:        router GEMM (fp32) -> moe_route (HIP) -> experts (HIP pair kernels or sorted segment GEMMs)
@@ -251,7 +252,7 @@ class TifepelModel:
                 m = spec.mixer
                 if m.conv > 1:
                     fields[f"conv.{r}"] = ((m.conv - 1, m.conv_channels), f32)
-                fields[f"ssm.{r}"] = ((m.heads, m.state, m.vdim), f32)
+                fields[f"ssm.{r}"] = ((m.heads, m.vdim, m.state), f32)
         return fields
 
     def attach_cache(self, pool, state_pool=None) -> None:
@@ -275,8 +276,15 @@ class TifepelModel:
             mix.masked_attn_rows(qkv[:nd], kc, vc, meta.dec_block_tables, None, meta.positions[:nd], m.heads,
                                  m.kv_heads, m.scale, 0, None, out=out[:nd], dist_bias=L.dist_bias)
         if meta.num_prefill_tokens > 0:
-            mix.masked_attn_rows(qkv[nd:], kc, vc, meta.pre_block_tables, meta.pre_cu_seqlens, meta.positions[nd:],
-                                 m.heads, m.kv_heads, m.scale, 0, None, out=out[nd:], dist_bias=L.dist_bias)
+            if (qkv.is_cuda and qkv.dtype == torch.bfloat16 and m.dim == m.vdim and m.dim in (64, 128)
+                    and qkv.shape[1] % 8 == 0 and mix.masked_prefill_available()):
+                # MFMA flash kernel (bf16 heads of 64 / 128 dims); other geometries and fp32: the row-wise kernel
+                mix.paged_prefill_masked(qkv[nd:], kc, vc, meta.pre_block_tables, meta.pre_cu_seqlens,
+                                         meta.pre_context_lens, m.heads, m.kv_heads, m.scale, 0, None,
+                                         tiles=meta.pre_tiles, out=out[nd:], dist_bias=L.dist_bias)
+            else:
+                mix.masked_attn_rows(qkv[nd:], kc, vc, meta.pre_block_tables, meta.pre_cu_seqlens, meta.positions[nd:],
+                                     m.heads, m.kv_heads, m.scale, 0, None, out=out[nd:], dist_bias=L.dist_bias)
         return ops.linear(out, L.o)
 
     def _unit(self, n: int) -> torch.Tensor:

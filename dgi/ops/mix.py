@@ -247,10 +247,11 @@ def masked_prefill_available() -> bool:
 
 
 def paged_prefill_masked(q, k_cache, v_cache, block_tables, cu_seqlens_q, context_lens, nh, nkv, scale,
-                         mask: int = 0, gate=None, tiles=None, out=None) -> torch.Tensor:
+                         mask: int = 0, gate=None, tiles=None, out=None, dist_bias=None) -> torch.Tensor:
     """``paged_prefill`` with a block mask — a query at position p sees keys
     [floor(p / mask) * mask, p] (``mask`` 0: all keys up to p) — and an optional sigmoid output
-    gate (out *= sigmoid(gate)).  bf16, key size == value size in {64, 128} on the GPU
+    gate (out *= sigmoid(gate)) and an optional distance bias (``dist_bias`` as in
+    ``masked_attn_rows``).  bf16, key size == value size in {64, 128} on the GPU
     (dgi/csrc/mix/masked_prefill.hip); the row-wise reference elsewhere."""
     from dgi import ops
     if _native(q):
@@ -261,13 +262,13 @@ def paged_prefill_masked(q, k_cache, v_cache, block_tables, cu_seqlens_q, contex
             tl = ops.prefill_tiles(cu_seqlens_q.tolist(), context_lens=context_lens.tolist(), tile=128)
             tiles = torch.tensor(tl if tl else [[0, 0]], dtype=torch.int32, device=q.device)[: len(tl)]
         _call("paged_prefill_masked", out, q, k_cache, v_cache, block_tables, cu_seqlens_q, context_lens, tiles,
-              nh, nkv, float(scale), int(mask), gate)
+              nh, nkv, float(scale), int(mask), gate, dist_bias)
         return out
     cu = cu_seqlens_q.tolist()
     pos = torch.cat([torch.arange(int(context_lens[b]) - (cu[b + 1] - cu[b]), int(context_lens[b]), dtype=torch.int32)
                      for b in range(len(cu) - 1)]) if len(cu) > 1 else torch.zeros(0, dtype=torch.int32)
     r = masked_attn_rows_ref(q, k_cache, v_cache, block_tables, cu_seqlens_q, pos.to(q.device), nh, nkv, scale,
-                             mask, gate)
+                             mask, gate, dist_bias)
     if out is not None:
         out.copy_(r)
         return out

@@ -8,8 +8,10 @@ and ``down`` [E, W, ff].
 
 Two evaluation paths on the GPU, same result up to summation order:
 
-* few rows (decode steps): one kernel pair walks the (token, route) pairs, each reading its
-  expert's rows straight from the stacked weights (weight-bandwidth bound, no host round trip);
+* few rows (decode steps, and every step inside a captured graph): workgroups own (expert, output
+  tile) and walk the pairs that chose the expert, so each expert's rows stream from the stacked
+  weights once per handful of tokens (weight-bandwidth bound, no host round trip), then the combine
+  kernel;
 * many rows (prompt portions): pairs are sorted by expert, every expert with tokens runs the
   vendor GEMM over its contiguous segment, and a combine kernel gathers each token's routes in
   their fixed order (deterministic, no atomics).
@@ -24,8 +26,8 @@ import torch
 
 from dgi.ops.mix import _call, _native
 
-# rows up to which the pair kernels evaluate the experts (above: sorted segments + GEMMs)
-PAIR_ROWS = int(os.environ.get("DGI_MOE_PAIR_ROWS", "32"))
+# rows up to which the expert-major kernels evaluate the experts (above: sorted segments + GEMMs)
+EXPERT_MAJOR_ROWS = int(os.environ.get("DGI_MOE_EXPERT_MAJOR_ROWS", "64"))
 
 
 def silu_mul_ref(gu: torch.Tensor) -> torch.Tensor:
@@ -86,10 +88,12 @@ def moe_experts(h, idx, wts, gate_up, down, shared=None) -> torch.Tensor:
     E, ff = gate_up.shape[0], down.shape[2]
     top = idx.shape[1]
     out = torch.empty(T, W, dtype=h.dtype, device=h.device)
-    if T <= PAIR_ROWS or torch.cuda.is_current_stream_capturing():
+    if T <= EXPERT_MAJOR_ROWS or torch.cuda.is_current_stream_capturing():
         mid = torch.empty(T * top, ff, dtype=torch.float32, device=h.device)
-        _call("moe_pair_gate_up", mid, h, idx, gate_up)
-        _call("moe_pair_down", out, mid, h, idx, wts, down, shared)
+        ys = torch.empty(T * top, W, dtype=h.dtype, device=h.device)     # identity pairs' rows are never read
+        _call("moe_expert_gate_up", mid, h, idx, gate_up)
+        _call("moe_expert_down", ys, mid, idx, down)
+        _call("moe_combine", out, ys, None, h, idx, wts, shared, E)
         return out
     from dgi import ops
     flat = idx.reshape(-1).long()

@@ -168,11 +168,11 @@ def ssm_scan_ref(xbc, dt_raw, dt_bias, a_log, d_skip, state, positions, seq_row0
     for r0, r1, slot, p0 in _seqs(positions, seq_row0, seq_slots):
         if r1 == r0:
             continue
-        S = torch.zeros(heads, N, dv) if p0 == 0 else state[slot].clone()
+        S = torch.zeros(heads, N, dv) if p0 == 0 else state[slot].transpose(1, 2).clone()
         for t in range(r0, r1):
             S = dA[t, :, None, None] * S + dt[t, :, None, None] * Bm[t, :, :, None] * x[t, :, None, :]
             y[t] = torch.einsum("hnv,hn->hv", S, Cm[t]) + d_skip[:, None] * x[t]
-        state[slot] = S
+        state[slot] = S.transpose(1, 2)
     return y.reshape(T, inner)
 
 
@@ -181,7 +181,7 @@ def ssm_scan(xbc, dt_raw, dt_bias, a_log, d_skip, state, positions, seq_row0, se
     """Mamba-2 recurrence over packed rows.  ``xbc`` [T, heads*dv + 2*G*N] fp32 = x | B | C (after the
     convolution), ``dt_raw`` [T, heads] the projected step sizes; per head h (group floor(h / (heads/G))):
     dt = softplus(dt_raw + dt_bias), S <- exp(-exp(a_log) dt) S + dt B x^T, y = S^T C + d_skip x, with
-    S [N, dv] in fp32 read from / written to ``state`` [slots, heads, N, dv] (zero at position 0).
+    S [N, dv] in fp32 read from / written to ``state`` [slots, heads, dv, N] (value-major; zero at position 0).
     Returns y [T, heads*dv] fp32."""
     if _native(xbc):
         y = torch.empty(xbc.shape[0], heads * dv, dtype=torch.float32, device=xbc.device)

@@ -299,7 +299,7 @@ def test_ssm_scan_portions_and_slots(device, dtype, geom):
     da[3], da[4] = 30.0, -30.0                     # softplus without overflow and without a clamp
     want_a = oracle_scan(xa, da[:, 1:1 + heads], dt_bias, a_log, d_skip, heads, dv, N, G)
     want_b = oracle_scan(xb, db[:, 1:1 + heads], dt_bias, a_log, d_skip, heads, dv, N, G)
-    state = torch.randn(6, heads, N, dv).to(device) * 50
+    state = torch.randn(6, heads, dv, N).to(device) * 50
     at_a = at_b = 0
     got_a, got_b = [], []
     for i, c in enumerate([1, 1, 2, 7, 1, 13, n]):
@@ -335,7 +335,7 @@ def test_scan_remembers_a_far_token(device, dtype):
     xbc[-1, dv + N] = 1.0                          # C_last = (1, 0, 0)
     dt_raw = torch.full((n, 1), -2.0).to(dtype)
     a_log = torch.tensor([-4.0])
-    state = torch.randn(3, heads, N, dv).to(device)
+    state = torch.randn(3, heads, dv, N).to(device)
     pos, _rs, r0, sl = seq_meta([200], [0], [1], device)
     args = (torch.zeros(1).to(device), a_log.to(device), torch.zeros(1).to(device), state)
     recur.ssm_scan(xbc[:200].to(device), dt_raw[:200].to(device), *args, pos, r0, sl, heads, dv, N, G)
@@ -412,9 +412,39 @@ def test_attention_temperature_bias_and_edges(device, dtype, geom):
     close(got, want[dec], tol)
 
 
+@pytest.mark.gpu
+@pytest.mark.parametrize("hd,H,G", [(64, 4, 2), (128, 8, 2)])
+def test_mfma_prompt_attention_with_distance_bias(hd, H, G):
+    """Prompt portions on the MFMA flash kernel (bf16 heads of 64 / 128 dims): a portion on top of a
+    cached prefix and a fresh prompt in one launch, a bias table that ends inside a 64-key tile and
+    one longer than the context, against the row-wise reference (fp32 math on the same bf16 cache)."""
+    from dgi import ops
+    g = torch.Generator().manual_seed(8)
+    bs, NB = 16, 64
+    lens, ctxs = [200, 77], [333, 77]              # rows of this step, context including them
+    T = sum(lens)
+    q = torch.randn(T, H * hd, generator=g).to(torch.bfloat16)
+    kc = torch.randn(NB, G, bs, hd, generator=g).to(torch.bfloat16)
+    vc = torch.randn(NB, G, bs, hd, generator=g).to(torch.bfloat16)
+    bt = torch.zeros(2, 24, dtype=I32)
+    bt[0, :21] = torch.arange(1, 22, dtype=I32)
+    bt[1, :5] = torch.arange(30, 35, dtype=I32)
+    cu = torch.tensor([0, 200, 277], dtype=I32)
+    ctx = torch.tensor(ctxs, dtype=I32)
+    pos = torch.cat([torch.arange(133, 333), torch.arange(0, 77)]).to(I32)
+    scale = hd ** -0.5
+    for rows, far in ((12, 100.0), (16, 1000.0)):
+        db = mix.distance_bias_table(torch.randn(rows, H, generator=g) * 2, far)
+        want = mix.masked_attn_rows_ref(q, kc, vc, bt, cu, pos, H, G, scale, 0, None, db)
+        tl = ops.prefill_tiles(cu.tolist(), context_lens=ctx.tolist(), tile=128)
+        got = mix.paged_prefill_masked(q.cuda(), kc.cuda(), vc.cuda(), bt.cuda(), cu.cuda(), ctx.cuda(), H, G, scale, 0, None,
+                                       tiles=torch.tensor(tl, dtype=I32).cuda(), dist_bias=db.cuda())
+        close(got, want, 3e-2)
+
+
 @pytest.mark.parametrize("device", DEVICES)
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("T,E,I,top", [(5, 6, 3, 3), (70, 6, 3, 3), (9, 4, 0, 1), (40, 2, 2, 4), (3, 70, 0, 8)])
+@pytest.mark.parametrize("T,E,I,top", [(5, 6, 3, 3), (70, 6, 3, 3), (9, 4, 0, 1), (40, 2, 2, 4), (3, 70, 0, 8), (300, 3, 1, 2)])
 def test_moe_routing_and_experts(device, dtype, T, E, I, top):
     g = torch.Generator().manual_seed(7)
     W, ff = 48, 20
