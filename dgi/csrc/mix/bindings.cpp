@@ -46,7 +46,8 @@ int dgi_causal_conv(void* out, int out_f32, const void* x, int x_f32, int x_stri
                     const int* seq_slots, int n_seq, int act, int residual, hipStream_t s);
 int dgi_ssm_scan(float* y, const float* xbc, int xbc_stride, const void* dt_raw, int dt_f32, int dt_stride,
                  const float* dt_bias, const float* a_log, const float* d_skip, float* state, const int* positions,
-                 const int* seq_row0, const int* seq_slots, int n_seq, int heads, int dv, int N, int G, hipStream_t s);
+                 const int* seq_row0, const int* seq_slots, int n_seq, int heads, int dv, int N, int G, float* ws,
+                 float* wsd, int L, int nchunks, hipStream_t s);
 int dgi_gated_group_norm(void* out, int out_f32, const float* y, const void* z, int z_f32, int z_stride, const float* w,
                          int T, int C, int groups, float eps, hipStream_t s);
 int dgi_moe_route(int* idx, float* wts, const float* logits, int l_stride, const float* corr, int T, int R, int top,
@@ -376,7 +377,8 @@ void causal_conv(at::Tensor out, const at::Tensor& x, const at::Tensor& w, const
 
 void ssm_scan(at::Tensor y, const at::Tensor& xbc, const at::Tensor& dt_raw, const at::Tensor& dt_bias,
               const at::Tensor& a_log, const at::Tensor& d_skip, at::Tensor state, const at::Tensor& positions,
-              const at::Tensor& seq_row0, const at::Tensor& seq_slots, int64_t heads, int64_t dv, int64_t N, int64_t G) {
+              const at::Tensor& seq_row0, const at::Tensor& seq_slots, int64_t heads, int64_t dv, int64_t N, int64_t G,
+              c10::optional<at::Tensor> ws, c10::optional<at::Tensor> wsd, int64_t L, int64_t nchunks) {
   check_f32(y, "y"); check_f32(xbc, "xbc"); check_f32(state, "state");
   const int df = act_kind(dt_raw, "dt_raw");
   check_rows(dt_raw, "dt_raw");
@@ -386,10 +388,19 @@ void ssm_scan(at::Tensor y, const at::Tensor& xbc, const at::Tensor& dt_raw, con
   TORCH_CHECK(state.dim() == 4 && state.size(1) == heads && state.size(2) == dv && state.size(3) == N, "state must be [slots, heads, dv, N]");
   check_f32(dt_bias, "dt_bias", heads); check_f32(a_log, "a_log", heads); check_f32(d_skip, "d_skip", heads);
   const int n_seq = (int)seq_slots.numel();
+  float *wsp = nullptr, *wdp = nullptr;
+  if (ws.has_value()) {
+    TORCH_CHECK(wsd.has_value() && L >= 1 && nchunks >= 1, "ssm_scan: the chunked form needs both workspaces");
+    check_f32(*ws, "ws", (int64_t)n_seq * nchunks * heads * dv * N);
+    check_f32(*wsd, "wsd", (int64_t)n_seq * nchunks * heads);
+    TORCH_CHECK(nchunks * L >= T, "ssm_scan: nchunks * L must cover the longest portion");
+    wsp = ws->data_ptr<float>(); wdp = wsd->data_ptr<float>();
+  }
   check_rc(dgi_ssm_scan(y.data_ptr<float>(), xbc.data_ptr<float>(), (int)xbc.stride(0), dt_raw.data_ptr(), df,
                         (int)dt_raw.stride(0), dt_bias.data_ptr<float>(), a_log.data_ptr<float>(), d_skip.data_ptr<float>(),
                         state.data_ptr<float>(), i32p(positions, "positions", T), i32p(seq_row0, "seq_row0", n_seq + 1),
-                        i32p(seq_slots, "seq_slots"), n_seq, (int)heads, (int)dv, (int)N, (int)G, cur_stream()), "ssm_scan");
+                        i32p(seq_slots, "seq_slots"), n_seq, (int)heads, (int)dv, (int)N, (int)G, wsp, wdp, (int)L,
+                        (int)nchunks, cur_stream()), "ssm_scan");
 }
 
 void gated_group_norm(at::Tensor out, const at::Tensor& y, const at::Tensor& z, const at::Tensor& w, int64_t groups,
@@ -496,7 +507,8 @@ TORCH_LIBRARY_FRAGMENT(dgi, m) {
   m.def("causal_conv(Tensor(a!) out, Tensor x, Tensor w, Tensor? bias, Tensor(b!)? tail, Tensor positions, Tensor row_seq, "
         "Tensor seq_row0, Tensor seq_slots, int act, bool residual) -> ()");
   m.def("ssm_scan(Tensor(a!) y, Tensor xbc, Tensor dt_raw, Tensor dt_bias, Tensor a_log, Tensor d_skip, Tensor(b!) state, "
-        "Tensor positions, Tensor seq_row0, Tensor seq_slots, int heads, int dv, int N, int G) -> ()");
+        "Tensor positions, Tensor seq_row0, Tensor seq_slots, int heads, int dv, int N, int G, Tensor(c!)? ws=None, "
+        "Tensor(d!)? wsd=None, int L=0, int nchunks=0) -> ()");
   m.def("gated_group_norm(Tensor(a!) out, Tensor y, Tensor z, Tensor w, int groups, float eps) -> ()");
   m.def("moe_route(Tensor(a!) idx, Tensor(b!) wts, Tensor logits, Tensor correction) -> ()");
   m.def("glu_silu(Tensor(a!) out, Tensor gu) -> ()");

@@ -26,6 +26,30 @@ template <typename T> __device__ __forceinline__ void stf(T* p, float v);
 template <> __device__ __forceinline__ void stf<float>(float* p, float v) { *p = v; }
 template <> __device__ __forceinline__ void stf<uint16_t>(uint16_t* p, float v) { *p = f32_to_bf16(v); }
 
+// 16 bytes of weights as floats: 8 bf16 or 4 fp32
+template <typename T> __device__ __forceinline__ void ld16(const T* p, float* f);
+template <> __device__ __forceinline__ void ld16<uint16_t>(const uint16_t* p, float* f) {
+  unpack8(*reinterpret_cast<const u32x4*>(p), f);
+}
+template <> __device__ __forceinline__ void ld16<float>(const float* p, float* f) {
+  const float4 v = *reinterpret_cast<const float4*>(p);
+  f[0] = v.x; f[1] = v.y; f[2] = v.z; f[3] = v.w;
+}
+
+// four consecutive weights as floats (8 bytes of bf16 or 16 of fp32): consecutive lanes then read
+// consecutive 16-byte LDS words of the staged activations, which is bank-conflict free (eight-element
+// chunks put lanes 32 bytes apart: an 8-way conflict)
+template <typename T> __device__ __forceinline__ void ld4(const T* p, float* f);
+template <> __device__ __forceinline__ void ld4<uint16_t>(const uint16_t* p, float* f) {
+  const uint2 v = *reinterpret_cast<const uint2*>(p);
+  f[0] = __uint_as_float(v.x << 16); f[1] = __uint_as_float(v.x & 0xffff0000u);
+  f[2] = __uint_as_float(v.y << 16); f[3] = __uint_as_float(v.y & 0xffff0000u);
+}
+template <> __device__ __forceinline__ void ld4<float>(const float* p, float* f) {
+  const float4 v = *reinterpret_cast<const float4*>(p);
+  f[0] = v.x; f[1] = v.y; f[2] = v.z; f[3] = v.w;
+}
+
 constexpr int MAXR = 8;      // routes per lane: R <= 512
 
 __global__ __launch_bounds__(64) void moe_route_kernel(int* __restrict__ idx, float* __restrict__ wts,
@@ -97,8 +121,8 @@ __global__ void silu_mul_kernel(T* __restrict__ out, const T* __restrict__ gu, i
 // group of PG pairs (once in all for a decode step with a handful of tokens per expert) instead of
 // once per pair.  The pairs of e are found by scanning idx and compacted into an LDS list (their
 // order there does not matter: every pair's result is independent).
-constexpr int CAP = 4096;    // pairs scanned per round
-constexpr int OPB = 32;      // outputs per workgroup (8 per wave)
+constexpr int CAP = 1024;    // pairs scanned per round
+constexpr int OPB = 4;       // outputs per workgroup (1 per wave)
 
 template <int PG>
 __device__ __forceinline__ int collect_pairs(const int* __restrict__ idx, int base, int P, int e, int* list, int* cnt) {
@@ -128,9 +152,27 @@ __global__ __launch_bounds__(256) void moe_expert_gate_up_kernel(
     for (int g0 = 0; g0 < n; g0 += PG) {
       const int np = min(PG, n - g0);
       __syncthreads();                                // the previous group's rows are fully read
-      for (int i = threadIdx.x; i < PG * W; i += 256) {
-        const int p = i / W, w = i - p * W;
-        hs[i] = p < np ? ldf<T>(h + (size_t)(list[g0 + p] / top) * h_stride + w) : 0.f;
+      {
+        constexpr int EV = 16 / sizeof(T);
+        if (W % EV == 0 && h_stride % EV == 0 && ((uintptr_t)h & 15) == 0) {   // 16-byte loads, several in flight
+          const int cpr = W / EV;
+#pragma unroll 4
+          for (int i = threadIdx.x; i < PG * cpr; i += 256) {
+            const int p = i / cpr, c = i - p * cpr;
+            float f[EV];
+#pragma unroll
+            for (int k = 0; k < EV; ++k) f[k] = 0.f;
+            if (p < np) ld16<T>(h + (size_t)(list[g0 + p] / top) * h_stride + c * EV, f);
+#pragma unroll
+            for (int k = 0; k < EV; k += 4)
+              *reinterpret_cast<float4*>(hs + (size_t)p * W + c * EV + k) = make_float4(f[k], f[k + 1], f[k + 2], f[k + 3]);
+          }
+        } else {
+          for (int i = threadIdx.x; i < PG * W; i += 256) {
+            const int p = i / W, w = i - p * W;
+            hs[i] = p < np ? ldf<T>(h + (size_t)(list[g0 + p] / top) * h_stride + w) : 0.f;
+          }
+        }
       }
       __syncthreads();
       for (int j = 0; j < OPB / 4; ++j) {
@@ -141,13 +183,28 @@ __global__ __launch_bounds__(256) void moe_expert_gate_up_kernel(
         float ag[PG], au[PG];
 #pragma unroll
         for (int p = 0; p < PG; ++p) ag[p] = au[p] = 0.f;
-        for (int w = lane; w < W; w += 64) {
-          const float a = ldf<T>(gp + w), b = ldf<T>(up + w);
+        if (W % 4 == 0 && ((uintptr_t)gate_up & 15) == 0) {
+#pragma unroll 8
+          for (int c = lane; c < W / 4; c += 64) {
+            float a[4], b[4];
+            ld4<T>(gp + c * 4, a);
+            ld4<T>(up + c * 4, b);
 #pragma unroll
-          for (int p = 0; p < PG; ++p) {
-            const float x = hs[p * W + w];
-            ag[p] += a * x;
-            au[p] += b * x;
+            for (int p = 0; p < PG; ++p) {
+              const float4 x = *reinterpret_cast<const float4*>(hs + p * W + c * 4);
+              ag[p] += a[0] * x.x + a[1] * x.y + a[2] * x.z + a[3] * x.w;
+              au[p] += b[0] * x.x + b[1] * x.y + b[2] * x.z + b[3] * x.w;
+            }
+          }
+        } else {
+          for (int w = lane; w < W; w += 64) {
+            const float a = ldf<T>(gp + w), b = ldf<T>(up + w);
+#pragma unroll
+            for (int p = 0; p < PG; ++p) {
+              const float x = hs[p * W + w];
+              ag[p] += a * x;
+              au[p] += b * x;
+            }
           }
         }
 #pragma unroll
@@ -177,9 +234,20 @@ __global__ __launch_bounds__(256) void moe_expert_down_kernel(
     for (int g0 = 0; g0 < n; g0 += PG) {
       const int np = min(PG, n - g0);
       __syncthreads();
-      for (int i = threadIdx.x; i < PG * ff; i += 256) {
-        const int p = i / ff, f = i - p * ff;
-        ms[i] = p < np ? mid[(size_t)list[g0 + p] * ff + f] : 0.f;
+      if (ff % 4 == 0) {
+        const int cpr = ff / 4;
+#pragma unroll 4
+        for (int i = threadIdx.x; i < PG * cpr; i += 256) {
+          const int p = i / cpr, c = i - p * cpr;
+          float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+          if (p < np) v = *reinterpret_cast<const float4*>(mid + (size_t)list[g0 + p] * ff + c * 4);
+          *reinterpret_cast<float4*>(ms + (size_t)p * ff + c * 4) = v;
+        }
+      } else {
+        for (int i = threadIdx.x; i < PG * ff; i += 256) {
+          const int p = i / ff, f = i - p * ff;
+          ms[i] = p < np ? mid[(size_t)list[g0 + p] * ff + f] : 0.f;
+        }
       }
       __syncthreads();
       for (int j = 0; j < OPB / 4; ++j) {
@@ -189,10 +257,23 @@ __global__ __launch_bounds__(256) void moe_expert_down_kernel(
         float acc[PG];
 #pragma unroll
         for (int p = 0; p < PG; ++p) acc[p] = 0.f;
-        for (int f = lane; f < ff; f += 64) {
-          const float a = ldf<T>(dp + f);
+        if (ff % 4 == 0 && ((uintptr_t)down & 15) == 0) {
+#pragma unroll 4
+          for (int c = lane; c < ff / 4; c += 64) {
+            float a[4];
+            ld4<T>(dp + c * 4, a);
 #pragma unroll
-          for (int p = 0; p < PG; ++p) acc[p] += a * ms[p * ff + f];
+            for (int p = 0; p < PG; ++p) {
+              const float4 x = *reinterpret_cast<const float4*>(ms + p * ff + c * 4);
+              acc[p] += a[0] * x.x + a[1] * x.y + a[2] * x.z + a[3] * x.w;
+            }
+          }
+        } else {
+          for (int f = lane; f < ff; f += 64) {
+            const float a = ldf<T>(dp + f);
+#pragma unroll
+            for (int p = 0; p < PG; ++p) acc[p] += a * ms[p * ff + f];
+          }
         }
 #pragma unroll
         for (int p = 0; p < PG; ++p) {

@@ -47,7 +47,8 @@ __global__ __launch_bounds__(COLS * NL) void ssm_scan_kernel(
     float* __restrict__ y, const float* __restrict__ xbc, int xbc_stride, const TD* __restrict__ dt_raw, int dt_stride,
     const float* __restrict__ dt_bias, const float* __restrict__ a_log, const float* __restrict__ d_skip,
     float* __restrict__ state, const int* __restrict__ positions, const int* __restrict__ seq_row0,
-    const int* __restrict__ seq_slots, int heads, int dv, int N, int G) {
+    const int* __restrict__ seq_slots, int heads, int dv, int N, int G, int mode, int L, int nchunks,
+    float* __restrict__ ws, float* __restrict__ wsd) {
   constexpr int NP = 64 * NQ;
   constexpr int PB = (TT * NP) / (COLS * NL);          // B (and C) values a thread stages per tile
   extern __shared__ __attribute__((aligned(16))) float sm[];
@@ -56,19 +57,26 @@ __global__ __launch_bounds__(COLS * NL) void ssm_scan_kernel(
   float* sX = sC + TT * NP;
   float* sDt = sX + TT * COLS;
   float* sDa = sDt + TT;
-  const int seq = blockIdx.x, h = blockIdx.y;
+  // mode 0: a workgroup runs a sequence's whole portion from its state slot and back.  Modes 1 and 3
+  // run one chunk of L rows (blockIdx.x = sequence * nchunks + chunk): 1 from a zero state into the
+  // workspace (no outputs; also the chunk's summed log decay), 3 from the workspace state into y.
+  const int seq = mode ? blockIdx.x / nchunks : blockIdx.x, h = blockIdx.y;
+  const int chunk = mode ? blockIdx.x - seq * nchunks : 0;
   const int tid = threadIdx.x;
   const int l = tid & (NL - 1), col = tid >> 4;
   const int v = blockIdx.z * COLS + col;
-  const int r0 = seq_row0[seq], r1 = seq_row0[seq + 1];
+  const int s0 = seq_row0[seq], s1 = seq_row0[seq + 1];
+  const int r0 = s0 + chunk * L, r1 = mode ? min(s1, r0 + L) : s1;
   if (r1 <= r0) return;
   const bool vok = v < dv;
   const int g = h / (heads / G);
   const int inner = heads * dv;
   const float* bp = xbc + inner + (size_t)g * N;
   const float* cp = bp + (size_t)G * N;
-  float* sp = state + (((size_t)seq_slots[seq] * heads + h) * dv + v) * N;     // state [slot][head][v][n]
-  const bool fresh = positions[r0] == 0;
+  float* sp = mode ? ws + (((size_t)blockIdx.x * heads + h) * dv + v) * N
+                   : state + (((size_t)seq_slots[seq] * heads + h) * dv + v) * N;     // [..][head][v][n]
+  const bool fresh = mode == 1 || (mode == 0 && positions[s0] == 0);
+  float ldec = 0.f;                                    // mode 1: sum of log decays (threads < TT)
   float S[NQ][4];
 #pragma unroll
   for (int q = 0; q < NQ; ++q)
@@ -110,6 +118,7 @@ __global__ __launch_bounds__(COLS * NL) void ssm_scan_kernel(
       const float dt = fmaxf(z, 0.f) + log1pf(expf(-fabsf(z)));
       sDt[tid] = dt;
       sDa[tid] = expf(na * dt);
+      if (t0 + tid < r1) ldec += na * dt;
     }
     __syncthreads();
     if (t0 + TT < r1) prefetch(t0 + TT);                 // in flight while this tile is consumed
@@ -128,12 +137,19 @@ __global__ __launch_bounds__(COLS * NL) void ssm_scan_kernel(
         S[q][3] = a * S[q][3] + b4.w * dx;
         acc += S[q][0] * c4.x + S[q][1] * c4.y + S[q][2] * c4.z + S[q][3] * c4.w;
       }
+      if (mode != 1) {                                   // mode 1: chunk states only, no outputs
 #pragma unroll
-      for (int o = NL / 2; o > 0; o >>= 1) acc += __shfl_xor(acc, o, 64);
-      if (l == 0 && vok) y[(size_t)(t0 + k) * inner + (size_t)h * dv + v] = acc + dsk * xv;
+        for (int o = NL / 2; o > 0; o >>= 1) acc += __shfl_xor(acc, o, 64);
+        if (l == 0 && vok) y[(size_t)(t0 + k) * inner + (size_t)h * dv + v] = acc + dsk * xv;
+      }
     }
   }
-  if (vok) {
+  if (mode == 1 && blockIdx.z == 0 && tid < TT) {      // TT lanes of wave 0
+#pragma unroll
+    for (int o = TT / 2; o > 0; o >>= 1) ldec += __shfl_xor(ldec, o, 64);
+    if (tid == 0) wsd[(size_t)blockIdx.x * heads + h] = ldec;
+  }
+  if (vok && mode != 3) {
 #pragma unroll
     for (int q = 0; q < NQ; ++q)
 #pragma unroll
@@ -142,6 +158,29 @@ __global__ __launch_bounds__(COLS * NL) void ssm_scan_kernel(
         if (n < N) sp[n] = S[q][j];
       }
   }
+}
+
+// Between the two chunk passes: per (sequence, head, state element) walk the chunks in order,
+// S_in[c] <- S;  S <- exp(logdecay[c]) * S + S_local[c], starting from the state slot (zero at
+// position 0); the workspace then holds every chunk's incoming state and the slot the final one.
+__global__ __launch_bounds__(256) void ssm_chunk_states_kernel(
+    float* __restrict__ ws, const float* __restrict__ wsd, float* __restrict__ state, const int* __restrict__ positions,
+    const int* __restrict__ seq_row0, const int* __restrict__ seq_slots, int heads, int per_head, int L, int nchunks) {
+  const int seq = blockIdx.x, h = blockIdx.y;
+  const int e = blockIdx.z * 256 + threadIdx.x;
+  if (e >= per_head) return;
+  const int s0 = seq_row0[seq], n = seq_row0[seq + 1] - s0;
+  if (n <= 0) return;
+  float* sp = state + ((size_t)seq_slots[seq] * heads + h) * per_head + e;
+  float S = positions[s0] == 0 ? 0.f : *sp;
+  const int nc = (n + L - 1) / L;
+  for (int c = 0; c < nc; ++c) {
+    float* wp = ws + (((size_t)seq * nchunks + c) * heads + h) * per_head + e;
+    const float loc = *wp;
+    *wp = S;
+    S = expf(wsd[((size_t)seq * nchunks + c) * heads + h]) * S + loc;
+  }
+  *sp = S;
 }
 
 template <typename TZ, typename TO>
@@ -172,26 +211,46 @@ __global__ __launch_bounds__(256) void gated_group_norm_kernel(
 
 }  // namespace
 
+// ws / wsd: workspace for the chunked form ([n_seq * nchunks][heads][dv][N] states and [n_seq * nchunks][heads]
+// log decays) or null: one pass, sequence by sequence.  The chunked form splits every portion into chunks
+// of L rows that run in parallel (local states from zero, a short serial pass over the chunk states, then
+// the outputs from each chunk's incoming state): twice the recurrence work, nchunks times the workgroups.
+// It reassociates the fp32 sums, so fp32 models keep the one-pass form.
 extern "C" int dgi_ssm_scan(float* y, const float* xbc, int xbc_stride, const void* dt_raw, int dt_f32, int dt_stride,
                             const float* dt_bias, const float* a_log, const float* d_skip, float* state,
                             const int* positions, const int* seq_row0, const int* seq_slots, int n_seq, int heads,
-                            int dv, int N, int G, hipStream_t s) {
+                            int dv, int N, int G, float* ws, float* wsd, int L, int nchunks, hipStream_t s) {
   if (n_seq == 0) return 0;
   if (G <= 0 || heads % G) return -2;
   if (N > 256 || N <= 0 || dv <= 0) return -3;
-  const dim3 grid(n_seq, heads, (dv + COLS - 1) / COLS);
-  if (heads > 65535 || grid.z > 65535) return -4;
-#define DGI_SCAN(TD, NQ)                                                                                                \
-  ssm_scan_kernel<TD, NQ><<<grid, COLS * NL, (size_t)(2 * TT * 64 * NQ + TT * COLS + 2 * TT) * 4, s>>>(                 \
-      y, xbc, xbc_stride, (const TD*)dt_raw, dt_stride, dt_bias, a_log, d_skip, state, positions, seq_row0, seq_slots, \
-      heads, dv, N, G)
+  if (ws && (L < 1 || nchunks < 1 || !wsd)) return -5;
+  if (heads > 65535 || (dv + COLS - 1) / COLS > 65535) return -4;
   const int nq = (N + 63) / 64;
-  if (dt_f32) {
-    if (nq <= 1) DGI_SCAN(float, 1); else if (nq <= 2) DGI_SCAN(float, 2); else DGI_SCAN(float, 4);
-  } else {
-    if (nq <= 1) DGI_SCAN(uint16_t, 1); else if (nq <= 2) DGI_SCAN(uint16_t, 2); else DGI_SCAN(uint16_t, 4);
-  }
+  auto launch = [&](int mode) {
+    const dim3 grid(mode ? n_seq * nchunks : n_seq, heads, (dv + COLS - 1) / COLS);
+#define DGI_SCAN(TD, NQ)                                                                                                \
+  ssm_scan_kernel<TD, NQ><<<grid, COLS * NL, (size_t)(2 * TT * 64 * NQ + TT * COLS + 2 * TT) * 4, s>>>(             \
+      y, xbc, xbc_stride, (const TD*)dt_raw, dt_stride, dt_bias, a_log, d_skip, state, positions, seq_row0, seq_slots, \
+      heads, dv, N, G, mode, L, nchunks, ws, wsd)
+    if (dt_f32) {
+      if (nq <= 1) DGI_SCAN(float, 1); else if (nq <= 2) DGI_SCAN(float, 2); else DGI_SCAN(float, 4);
+    } else {
+      if (nq <= 1) DGI_SCAN(uint16_t, 1); else if (nq <= 2) DGI_SCAN(uint16_t, 2); else DGI_SCAN(uint16_t, 4);
+    }
 #undef DGI_SCAN
+  };
+  if (!ws) {
+    launch(0);
+    DGI_CHECK_LAUNCH();
+    return 0;
+  }
+  launch(1);
+  DGI_CHECK_LAUNCH();
+  const int per_head = dv * N;
+  ssm_chunk_states_kernel<<<dim3(n_seq, heads, (per_head + 255) / 256), 256, 0, s>>>(ws, wsd, state, positions, seq_row0,
+                                                                                      seq_slots, heads, per_head, L, nchunks);
+  DGI_CHECK_LAUNCH();
+  launch(3);
   DGI_CHECK_LAUNCH();
   return 0;
 }

@@ -12,6 +12,7 @@ state tensors (``dgi.kv.state_pool``).  A portion that starts at position 0 read
 """
 from __future__ import annotations
 
+import os
 from typing import Optional
 
 import torch
@@ -176,15 +177,40 @@ def ssm_scan_ref(xbc, dt_raw, dt_bias, a_log, d_skip, state, positions, seq_row0
     return y.reshape(T, inner)
 
 
+SCAN_CHUNK = int(os.environ.get("DGI_SCAN_CHUNK", "128"))       # rows per chunk of the chunked scan (0: off)
+SCAN_WS_BYTES = 512 << 20                                      # largest chunk-state workspace
+SCAN_CHUNK_BELOW = int(os.environ.get("DGI_SCAN_CHUNK_BELOW", "512"))   # one-pass workgroups below which steps are chunked
+
+
 def ssm_scan(xbc, dt_raw, dt_bias, a_log, d_skip, state, positions, seq_row0, seq_slots, heads: int, dv: int,
-             N: int, G: int) -> torch.Tensor:
+             N: int, G: int, chunked=None) -> torch.Tensor:
     """Mamba-2 recurrence over packed rows.  ``xbc`` [T, heads*dv + 2*G*N] fp32 = x | B | C (after the
     convolution), ``dt_raw`` [T, heads] the projected step sizes; per head h (group floor(h / (heads/G))):
     dt = softplus(dt_raw + dt_bias), S <- exp(-exp(a_log) dt) S + dt B x^T, y = S^T C + d_skip x, with
     S [N, dv] in fp32 read from / written to ``state`` [slots, heads, dv, N] (value-major; zero at position 0).
-    Returns y [T, heads*dv] fp32."""
+    Returns y [T, heads*dv] fp32.
+
+    On the GPU a step with long portions of few sequences runs in chunks of ``SCAN_CHUNK`` rows in
+    parallel (local chunk states, a serial pass over them, outputs from each chunk's incoming state)
+    when the model is bf16 (``chunked`` None) — the same recurrence with its fp32 sums reassociated;
+    fp32 models, short steps and steps with enough sequences to fill the chip run each sequence in one pass."""
     if _native(xbc):
-        y = torch.empty(xbc.shape[0], heads * dv, dtype=torch.float32, device=xbc.device)
+        T, n_seq = xbc.shape[0], seq_slots.shape[0]
+        y = torch.empty(T, heads * dv, dtype=torch.float32, device=xbc.device)
+        longest = T - n_seq + 1                       # no portion is longer (every sequence has a row)
+        L = SCAN_CHUNK
+        if chunked is None:
+            # worth twice the recurrence work only while one-pass workgroups (sequence x head x 16 columns)
+            # cannot fill the chip: measured slower than one pass from 512 workgroups on
+            chunked = dt_raw.dtype != torch.float32 and n_seq * heads * -(-dv // 16) < SCAN_CHUNK_BELOW
+        if chunked and L > 0 and longest >= 4 * L:
+            nch = -(-longest // L)
+            if n_seq * nch * heads * dv * N * 4 <= SCAN_WS_BYTES:
+                ws = torch.empty(n_seq * nch * heads * dv * N, dtype=torch.float32, device=xbc.device)
+                wsd = torch.empty(n_seq * nch * heads, dtype=torch.float32, device=xbc.device)
+                _call("ssm_scan", y, xbc, dt_raw, dt_bias, a_log, d_skip, state, positions, seq_row0, seq_slots,
+                      heads, dv, N, G, ws, wsd, L, nch)
+                return y
         _call("ssm_scan", y, xbc, dt_raw, dt_bias, a_log, d_skip, state, positions, seq_row0, seq_slots, heads, dv, N, G)
         return y
     return ssm_scan_ref(xbc, dt_raw, dt_bias, a_log, d_skip, state, positions, seq_row0, seq_slots, heads, dv, N, G)

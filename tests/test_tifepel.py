@@ -323,6 +323,32 @@ def test_ssm_scan_portions_and_slots(device, dtype, geom):
     close(torch.cat(got_b, 0), want_b[:at_b], 2e-5 * max(1.0, want_b.abs().max().item()))
 
 
+@pytest.mark.gpu
+@pytest.mark.parametrize("geom", [(4, 24, 20, 2), (2, 16, 130, 1)])
+def test_chunked_scan_equals_one_pass(geom, monkeypatch):
+    """The chunk-parallel form (local chunk states, serial pass over them, outputs per chunk) against
+    the oracle: portions that end inside a chunk, a one-row sequence beside them, a continued sequence
+    whose slot holds its state, and a fresh one whose slot holds garbage."""
+    heads, dv, N, G = geom
+    monkeypatch.setattr(recur, "SCAN_CHUNK", 16)
+    g = torch.Generator().manual_seed(9)
+    n = 150
+    xa, da, dt_bias, a_log, d_skip = mamba_parts(g, heads, dv, N, G, n, torch.float32)
+    xb, db = mamba_parts(g, heads, dv, N, G, n, torch.float32)[:2]
+    want_a = oracle_scan(xa, da[:, 1:1 + heads], dt_bias, a_log, d_skip, heads, dv, N, G)
+    want_b = oracle_scan(xb, db[:, 1:1 + heads], dt_bias, a_log, d_skip, heads, dv, N, G)
+    state = torch.randn(6, heads, dv, N).cuda() * 50
+    par = [t.cuda() for t in (dt_bias, a_log, d_skip)]
+    # step 1: a[0:70] (fresh) beside b[0:1]; step 2: a[70:150] (continued) beside b[1:131]
+    for (a0, a1, b0, b1) in ((0, 70, 0, 1), (70, 150, 1, 131)):
+        pos, _rs, r0, sl = seq_meta([a1 - a0, b1 - b0], [a0, b0], [2, 4], "cuda")
+        x = torch.cat([xa[a0:a1], xb[b0:b1]], 0).cuda()
+        d = torch.cat([da[a0:a1], db[b0:b1]], 0).cuda()[:, 1:1 + heads]
+        y = recur.ssm_scan(x, d, *par, state, pos, r0, sl, heads, dv, N, G, chunked=True)
+        close(y[: a1 - a0], want_a[a0:a1], 3e-5 * max(1.0, want_a.abs().max().item()))
+        close(y[a1 - a0:], want_b[b0:b1], 3e-5 * max(1.0, want_b.abs().max().item()))
+
+
 @pytest.mark.parametrize("device", DEVICES)
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_scan_remembers_a_far_token(device, dtype):
