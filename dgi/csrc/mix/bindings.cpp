@@ -469,7 +469,8 @@ void moe_combine(at::Tensor out, const at::Tensor& ys, const c10::optional<at::T
   const int T = (int)h.size(0), W = (int)h.size(1);
   TORCH_CHECK(act_kind(out, "out") == f && out.is_contiguous() && out.size(0) == T && out.size(1) == W);
   TORCH_CHECK(act_kind(ys, "ys") == f && ys.is_contiguous() && ys.dim() == 2 && ys.size(1) == W);
-  TORCH_CHECK(idx.dim() == 2 && idx.size(0) == T && wts.sizes() == idx.sizes() && ys.size(0) == idx.numel());
+  TORCH_CHECK(idx.dim() == 2 && idx.size(0) == T && wts.sizes() == idx.sizes());
+  TORCH_CHECK(where.has_value() || ys.size(0) == idx.numel(), "moe_combine: without `where` ys holds one row per pair");
   const void* sp = nullptr;
   int ss = 0;
   if (shared.has_value()) {

@@ -54,6 +54,67 @@ __global__ __launch_bounds__(256) void causal_conv_kernel(
   stf<TO>(out + (size_t)row * C + c, acc);
 }
 
+// Four channels per thread: 16-byte (fp32) / 8-byte (bf16) row accesses and the thread's 4 x taps
+// weights as contiguous 16-byte loads.  Same arithmetic, per channel, in the same order.
+template <typename T> __device__ __forceinline__ void ld4(const T* p, float* f);
+template <> __device__ __forceinline__ void ld4<float>(const float* p, float* f) {
+  const float4 v = *reinterpret_cast<const float4*>(p);
+  f[0] = v.x; f[1] = v.y; f[2] = v.z; f[3] = v.w;
+}
+template <> __device__ __forceinline__ void ld4<uint16_t>(const uint16_t* p, float* f) {
+  const uint2 v = *reinterpret_cast<const uint2*>(p);
+  f[0] = __uint_as_float(v.x << 16); f[1] = __uint_as_float(v.x & 0xffff0000u);
+  f[2] = __uint_as_float(v.y << 16); f[3] = __uint_as_float(v.y & 0xffff0000u);
+}
+template <typename T> __device__ __forceinline__ void st4(T* p, const float* f);
+template <> __device__ __forceinline__ void st4<float>(float* p, const float* f) {
+  *reinterpret_cast<float4*>(p) = make_float4(f[0], f[1], f[2], f[3]);
+}
+template <> __device__ __forceinline__ void st4<uint16_t>(uint16_t* p, const float* f) {
+  *reinterpret_cast<uint2*>(p) = make_uint2(pack_bf16x2(f[0], f[1]), pack_bf16x2(f[2], f[3]));
+}
+
+template <typename TI, typename TO, int TAPS>
+__global__ __launch_bounds__(256) void causal_conv_vec_kernel(
+    TO* __restrict__ out, const TI* __restrict__ x, int x_stride, int C, const float* __restrict__ w,
+    const float* __restrict__ bias, const float* __restrict__ tail, const int* __restrict__ positions,
+    const int* __restrict__ row_seq, const int* __restrict__ seq_row0, const int* __restrict__ seq_slots, int act,
+    int residual) {
+  const int row = blockIdx.x;
+  const int c = (blockIdx.y * blockDim.x + threadIdx.x) * 4;
+  if (c >= C) return;
+  const int seq = row_seq[row];
+  const int r0 = seq_row0[seq];
+  const int pos = positions[row], p0 = positions[r0];
+  const float* tl = tail ? tail + (size_t)seq_slots[seq] * (TAPS - 1) * C : nullptr;
+  float wv[4 * TAPS];
+#pragma unroll
+  for (int i = 0; i < TAPS; ++i) ld4<float>(w + (size_t)c * TAPS + 4 * i, wv + 4 * i);     // wv[ch * TAPS + j]
+  float acc[4] = {0.f, 0.f, 0.f, 0.f};
+  if (bias) ld4<float>(bias + c, acc);
+  float cur[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int j = 0; j < TAPS; ++j) {
+    const int pp = pos - (TAPS - 1) + j;
+    if (pp < 0) continue;
+    float v[4];
+    if (pp >= p0) ld4<TI>(x + (size_t)(r0 + pp - p0) * x_stride + c, v);
+    else ld4<float>(tl + (size_t)(pp - (p0 - (TAPS - 1))) * C + c, v);
+#pragma unroll
+    for (int ch = 0; ch < 4; ++ch) acc[ch] += wv[ch * TAPS + j] * v[ch];
+    if (j == TAPS - 1) {
+#pragma unroll
+      for (int ch = 0; ch < 4; ++ch) cur[ch] = v[ch];
+    }
+  }
+#pragma unroll
+  for (int ch = 0; ch < 4; ++ch) {
+    if (act == 1) acc[ch] = acc[ch] / (1.f + expf(-acc[ch]));
+    if (residual) acc[ch] += cur[ch];
+  }
+  st4<TO>(out + (size_t)row * C + c, acc);
+}
+
 template <typename TI>
 __global__ __launch_bounds__(256) void conv_tail_kernel(
     float* __restrict__ tail, const TI* __restrict__ x, int x_stride, int C, int taps, const int* __restrict__ positions,
@@ -91,6 +152,23 @@ extern "C" int dgi_causal_conv(void* out, int out_f32, const void* x, int x_f32,
   if (taps > 1 && !tail) return -3;
   const dim3 grid(T, (C + 255) / 256);
   if (grid.y > 65535) return -4;
+  // vector path: channels in fours, rows and tables 16-byte aligned
+  const bool vec = C % 4 == 0 && x_stride % 4 == 0 && taps >= 2 && taps <= 4 &&
+                   (((uintptr_t)x | (uintptr_t)out | (uintptr_t)w | (uintptr_t)bias | (uintptr_t)tail) & 15) == 0;
+  if (vec) {
+    const dim3 vgrid(T, (C / 4 + 255) / 256);
+#define DGI_CONVV(TI, TO, TP)                                                                                      \
+  causal_conv_vec_kernel<TI, TO, TP><<<vgrid, 256, 0, s>>>((TO*)out, (const TI*)x, x_stride, C, w, bias, tail,     \
+                                                          positions, row_seq, seq_row0, seq_slots, act, residual)
+#define DGI_CONVT(TI, TO) \
+  do { if (taps == 2) DGI_CONVV(TI, TO, 2); else if (taps == 3) DGI_CONVV(TI, TO, 3); else DGI_CONVV(TI, TO, 4); } while (0)
+    if (x_f32 && out_f32) DGI_CONVT(float, float);
+    else if (x_f32) DGI_CONVT(float, uint16_t);
+    else if (out_f32) DGI_CONVT(uint16_t, float);
+    else DGI_CONVT(uint16_t, uint16_t);
+#undef DGI_CONVT
+#undef DGI_CONVV
+  } else {
 #define DGI_CONV(TI, TO)                                                                                           \
   causal_conv_kernel<TI, TO><<<grid, 256, 0, s>>>((TO*)out, (const TI*)x, x_stride, C, taps, w, bias, tail, positions, \
                                                   row_seq, seq_row0, seq_slots, act, residual)
@@ -99,6 +177,7 @@ extern "C" int dgi_causal_conv(void* out, int out_f32, const void* x, int x_f32,
   else if (out_f32) DGI_CONV(uint16_t, float);
   else DGI_CONV(uint16_t, uint16_t);
 #undef DGI_CONV
+  }
   DGI_CHECK_LAUNCH();
   if (taps > 1) {
     const dim3 g2(n_seq, (C + 255) / 256);

@@ -105,13 +105,32 @@ __global__ __launch_bounds__(64) void moe_route_kernel(int* __restrict__ idx, fl
   }
 }
 
-template <typename T>
+template <typename T> __device__ __forceinline__ void st4(T* p, const float* f);
+template <> __device__ __forceinline__ void st4<float>(float* p, const float* f) {
+  *reinterpret_cast<float4*>(p) = make_float4(f[0], f[1], f[2], f[3]);
+}
+template <> __device__ __forceinline__ void st4<uint16_t>(uint16_t* p, const float* f) {
+  *reinterpret_cast<uint2*>(p) = make_uint2(pack_bf16x2(f[0], f[1]), pack_bf16x2(f[2], f[3]));
+}
+
+// V = 4: four columns per thread (I, the row stride and the pointers allow 8 / 16-byte accesses)
+template <typename T, int V>
 __global__ void silu_mul_kernel(T* __restrict__ out, const T* __restrict__ gu, int gu_stride, int rows, int I) {
-  const size_t n = (size_t)rows * I;
+  const size_t n = (size_t)rows * (I / V);
   for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) {
-    const size_t r = i / I, c = i - r * I;
-    const float g = ldf<T>(gu + r * gu_stride + c), u = ldf<T>(gu + r * gu_stride + I + c);
-    stf<T>(out + i, g / (1.f + expf(-g)) * u);
+    const size_t r = i / (I / V), c = (i - r * (I / V)) * V;
+    float g[V], u[V], o[V];
+    if constexpr (V == 4) {
+      ld4<T>(gu + r * gu_stride + c, g);
+      ld4<T>(gu + r * gu_stride + I + c, u);
+    } else {
+      g[0] = ldf<T>(gu + r * gu_stride + c);
+      u[0] = ldf<T>(gu + r * gu_stride + I + c);
+    }
+#pragma unroll
+    for (int k = 0; k < V; ++k) o[k] = g[k] / (1.f + expf(-g[k])) * u[k];
+    if constexpr (V == 4) st4<T>(out + r * I + c, o);
+    else stf<T>(out + r * I + c, o[0]);
   }
 }
 
@@ -141,8 +160,8 @@ __global__ __launch_bounds__(256) void moe_expert_gate_up_kernel(
     float* __restrict__ mid, const T* __restrict__ h, int h_stride, const int* __restrict__ idx,
     const T* __restrict__ gate_up, int P, int top, int ff, int W) {
   extern __shared__ __attribute__((aligned(16))) float sm[];
-  float* hs = sm;                                     // [PG][W]
-  int* list = reinterpret_cast<int*>(sm + (size_t)PG * W);   // [CAP]
+  int* list = reinterpret_cast<int*>(sm);             // [CAP]
+  T* hs = reinterpret_cast<T*>(sm + CAP);             // [PG][W] in the activation dtype (no rounding: h has it)
   __shared__ int cnt;
   const int e = blockIdx.x;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
@@ -154,23 +173,19 @@ __global__ __launch_bounds__(256) void moe_expert_gate_up_kernel(
       __syncthreads();                                // the previous group's rows are fully read
       {
         constexpr int EV = 16 / sizeof(T);
-        if (W % EV == 0 && h_stride % EV == 0 && ((uintptr_t)h & 15) == 0) {   // 16-byte loads, several in flight
+        if (W % EV == 0 && h_stride % EV == 0 && ((uintptr_t)h & 15) == 0) {   // 16-byte copies, several in flight
           const int cpr = W / EV;
 #pragma unroll 4
           for (int i = threadIdx.x; i < PG * cpr; i += 256) {
             const int p = i / cpr, c = i - p * cpr;
-            float f[EV];
-#pragma unroll
-            for (int k = 0; k < EV; ++k) f[k] = 0.f;
-            if (p < np) ld16<T>(h + (size_t)(list[g0 + p] / top) * h_stride + c * EV, f);
-#pragma unroll
-            for (int k = 0; k < EV; k += 4)
-              *reinterpret_cast<float4*>(hs + (size_t)p * W + c * EV + k) = make_float4(f[k], f[k + 1], f[k + 2], f[k + 3]);
+            u32x4 v = {0u, 0u, 0u, 0u};
+            if (p < np) v = *reinterpret_cast<const u32x4*>(h + (size_t)(list[g0 + p] / top) * h_stride + c * EV);
+            *reinterpret_cast<u32x4*>(hs + (size_t)p * W + c * EV) = v;
           }
         } else {
           for (int i = threadIdx.x; i < PG * W; i += 256) {
             const int p = i / W, w = i - p * W;
-            hs[i] = p < np ? ldf<T>(h + (size_t)(list[g0 + p] / top) * h_stride + w) : 0.f;
+            hs[i] = p < np ? h[(size_t)(list[g0 + p] / top) * h_stride + w] : T(0);
           }
         }
       }
@@ -191,9 +206,10 @@ __global__ __launch_bounds__(256) void moe_expert_gate_up_kernel(
             ld4<T>(up + c * 4, b);
 #pragma unroll
             for (int p = 0; p < PG; ++p) {
-              const float4 x = *reinterpret_cast<const float4*>(hs + p * W + c * 4);
-              ag[p] += a[0] * x.x + a[1] * x.y + a[2] * x.z + a[3] * x.w;
-              au[p] += b[0] * x.x + b[1] * x.y + b[2] * x.z + b[3] * x.w;
+              float x[4];
+              ld4<T>(hs + p * W + c * 4, x);
+              ag[p] += a[0] * x[0] + a[1] * x[1] + a[2] * x[2] + a[3] * x[3];
+              au[p] += b[0] * x[0] + b[1] * x[1] + b[2] * x[2] + b[3] * x[3];
             }
           }
         } else {
@@ -201,7 +217,7 @@ __global__ __launch_bounds__(256) void moe_expert_gate_up_kernel(
             const float a = ldf<T>(gp + w), b = ldf<T>(up + w);
 #pragma unroll
             for (int p = 0; p < PG; ++p) {
-              const float x = hs[p * W + w];
+              const float x = ldf<T>(hs + p * W + w);
               ag[p] += a * x;
               au[p] += b * x;
             }
@@ -224,8 +240,8 @@ __global__ __launch_bounds__(256) void moe_expert_down_kernel(
     T* __restrict__ ys, const float* __restrict__ mid, const int* __restrict__ idx, const T* __restrict__ down, int P,
     int ff, int W) {
   extern __shared__ __attribute__((aligned(16))) float sm[];
-  float* ms = sm;                                     // [PG][ff]
-  int* list = reinterpret_cast<int*>(sm + (size_t)PG * ff);
+  int* list = reinterpret_cast<int*>(sm);             // [CAP]
+  float* ms = sm + CAP;                               // [PG][ff]
   __shared__ int cnt;
   const int e = blockIdx.x;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
@@ -286,22 +302,33 @@ __global__ __launch_bounds__(256) void moe_expert_down_kernel(
   }
 }
 
-template <typename T>
+template <typename T, int V>
 __global__ __launch_bounds__(256) void moe_combine_kernel(
     T* __restrict__ out, const T* __restrict__ ys, const int* __restrict__ where, const T* __restrict__ h, int h_stride,
     const int* __restrict__ idx, const float* __restrict__ wts, const T* __restrict__ shared, int shared_stride, int E,
     int top, int W) {
   const int t = blockIdx.x;
-  const int w = blockIdx.y * 256 + threadIdx.x;
+  const int w = (blockIdx.y * 256 + threadIdx.x) * V;
   if (w >= W) return;
-  float acc = shared ? ldf<T>(shared + (size_t)t * shared_stride + w) : 0.f;
+  float acc[V], v[V];
+#pragma unroll
+  for (int k = 0; k < V; ++k) acc[k] = 0.f;
+  if (shared) {
+    if constexpr (V == 4) ld4<T>(shared + (size_t)t * shared_stride + w, acc);
+    else acc[0] = ldf<T>(shared + (size_t)t * shared_stride + w);
+  }
   for (int k = 0; k < top; ++k) {
     const int e = idx[(size_t)t * top + k];
     const float wt = wts[(size_t)t * top + k];
-    if (e >= E || e < 0) acc += wt * ldf<T>(h + (size_t)t * h_stride + w);
-    else acc += wt * ldf<T>(ys + (size_t)(where ? where[(size_t)t * top + k] : t * top + k) * W + w);
+    const T* src = (e >= E || e < 0) ? h + (size_t)t * h_stride + w
+                                     : ys + (size_t)(where ? where[(size_t)t * top + k] : t * top + k) * W + w;
+    if constexpr (V == 4) ld4<T>(src, v);
+    else v[0] = ldf<T>(src);
+#pragma unroll
+    for (int j = 0; j < V; ++j) acc[j] += wt * v[j];
   }
-  stf<T>(out + (size_t)t * W + w, acc);
+  if constexpr (V == 4) st4<T>(out + (size_t)t * W + w, acc);
+  else stf<T>(out + (size_t)t * W + w, acc[0]);
 }
 
 }  // namespace
@@ -317,31 +344,49 @@ extern "C" int dgi_moe_route(int* idx, float* wts, const float* logits, int l_st
 
 extern "C" int dgi_glu_silu(void* out, const void* gu, int gu_stride, int rows, int I, int is_f32, hipStream_t s) {
   if (rows == 0 || I == 0) return 0;
-  const size_t n = (size_t)rows * I;
+  const bool vec = I % 4 == 0 && gu_stride % 4 == 0 && (((uintptr_t)out | (uintptr_t)gu) & 15) == 0;
+  const size_t n = (size_t)rows * (vec ? I / 4 : I);
   const int blocks = (int)((n + 255) / 256 > 65535 ? 65535 : (n + 255) / 256);
-  if (is_f32) silu_mul_kernel<float><<<blocks, 256, 0, s>>>((float*)out, (const float*)gu, gu_stride, rows, I);
-  else silu_mul_kernel<uint16_t><<<blocks, 256, 0, s>>>((uint16_t*)out, (const uint16_t*)gu, gu_stride, rows, I);
+  if (is_f32) {
+    if (vec) silu_mul_kernel<float, 4><<<blocks, 256, 0, s>>>((float*)out, (const float*)gu, gu_stride, rows, I);
+    else silu_mul_kernel<float, 1><<<blocks, 256, 0, s>>>((float*)out, (const float*)gu, gu_stride, rows, I);
+  } else {
+    if (vec) silu_mul_kernel<uint16_t, 4><<<blocks, 256, 0, s>>>((uint16_t*)out, (const uint16_t*)gu, gu_stride, rows, I);
+    else silu_mul_kernel<uint16_t, 1><<<blocks, 256, 0, s>>>((uint16_t*)out, (const uint16_t*)gu, gu_stride, rows, I);
+  }
   DGI_CHECK_LAUNCH();
   return 0;
 }
 
-// pairs per group by LDS budget (PG rows of `row_len` floats + the pair list within 64 KiB)
-static int pick_pg(int row_len) {
-  const int room = (64 * 1024 - CAP * 4) / 4;
-  return row_len * 8 <= room ? 8 : (row_len * 4 <= room ? 4 : (row_len * 2 <= room ? 2 : (row_len <= room ? 1 : 0)));
+// pairs per group by LDS budget: PG rows of `row_bytes` + the pair list within 96 KiB (two workgroups a CU)
+static int pick_pg(size_t row_bytes) {
+  const size_t room = 96 * 1024 - CAP * 4;
+  return row_bytes * 8 <= room ? 8 : (row_bytes * 4 <= room ? 4 : (row_bytes * 2 <= room ? 2 : (row_bytes <= room ? 1 : 0)));
+}
+
+// more than 64 KiB of dynamic LDS has to be allowed per kernel, once
+template <typename K>
+static int allow_lds(K kernel, size_t lds) {
+  if (lds <= 64 * 1024) return 0;
+  return (int)hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
 }
 
 extern "C" int dgi_moe_expert_gate_up(float* mid, const void* h, int h_stride, const int* idx, const void* gate_up,
                                       int T, int E, int top, int ff, int W, int is_f32, hipStream_t s) {
   if (T == 0 || E == 0) return 0;
-  const int pg = pick_pg(W);
+  const size_t es = is_f32 ? 4 : 2;
+  const int pg = pick_pg((size_t)W * es);
   if (!pg) return -2;
   const dim3 grid(E, (ff + OPB - 1) / OPB);
   if (grid.y > 65535) return -3;
-  const size_t lds = ((size_t)pg * W + CAP) * 4;
-#define DGI_GU(TT_, PG_)                                                                                   \
-  moe_expert_gate_up_kernel<TT_, PG_><<<grid, 256, lds, s>>>(mid, (const TT_*)h, h_stride, idx, (const TT_*)gate_up, \
-                                                            T * top, top, ff, W)
+  const size_t lds = (size_t)pg * W * es + CAP * 4;
+#define DGI_GU(TT_, PG_)                                                                                        \
+  do {                                                                                                          \
+    static const int ok = allow_lds(moe_expert_gate_up_kernel<TT_, PG_>, 96 * 1024);                            \
+    if (ok != 0) return ok;                                                                                     \
+    moe_expert_gate_up_kernel<TT_, PG_><<<grid, 256, lds, s>>>(mid, (const TT_*)h, h_stride, idx, (const TT_*)gate_up, \
+                                                              T * top, top, ff, W);                             \
+  } while (0)
   if (is_f32) { if (pg == 8) DGI_GU(float, 8); else if (pg == 4) DGI_GU(float, 4); else if (pg == 2) DGI_GU(float, 2); else DGI_GU(float, 1); }
   else { if (pg == 8) DGI_GU(uint16_t, 8); else if (pg == 4) DGI_GU(uint16_t, 4); else if (pg == 2) DGI_GU(uint16_t, 2); else DGI_GU(uint16_t, 1); }
 #undef DGI_GU
@@ -352,13 +397,17 @@ extern "C" int dgi_moe_expert_gate_up(float* mid, const void* h, int h_stride, c
 extern "C" int dgi_moe_expert_down(void* ys, const float* mid, const int* idx, const void* down, int T, int E, int top,
                                    int ff, int W, int is_f32, hipStream_t s) {
   if (T == 0 || E == 0) return 0;
-  const int pg = pick_pg(ff);
+  const int pg = pick_pg((size_t)ff * 4);
   if (!pg) return -2;
   const dim3 grid(E, (W + OPB - 1) / OPB);
   if (grid.y > 65535) return -3;
   const size_t lds = ((size_t)pg * ff + CAP) * 4;
-#define DGI_DN(TT_, PG_) \
-  moe_expert_down_kernel<TT_, PG_><<<grid, 256, lds, s>>>((TT_*)ys, mid, idx, (const TT_*)down, T * top, ff, W)
+#define DGI_DN(TT_, PG_)                                                                                         \
+  do {                                                                                                           \
+    static const int ok = allow_lds(moe_expert_down_kernel<TT_, PG_>, 96 * 1024);                                \
+    if (ok != 0) return ok;                                                                                      \
+    moe_expert_down_kernel<TT_, PG_><<<grid, 256, lds, s>>>((TT_*)ys, mid, idx, (const TT_*)down, T * top, ff, W); \
+  } while (0)
   if (is_f32) { if (pg == 8) DGI_DN(float, 8); else if (pg == 4) DGI_DN(float, 4); else if (pg == 2) DGI_DN(float, 2); else DGI_DN(float, 1); }
   else { if (pg == 8) DGI_DN(uint16_t, 8); else if (pg == 4) DGI_DN(uint16_t, 4); else if (pg == 2) DGI_DN(uint16_t, 2); else DGI_DN(uint16_t, 1); }
 #undef DGI_DN
@@ -370,14 +419,16 @@ extern "C" int dgi_moe_combine(void* out, const void* ys, const int* where, cons
                                const float* wts, const void* shared, int shared_stride, int T, int E, int top, int W,
                                int is_f32, hipStream_t s) {
   if (T == 0) return 0;
-  const dim3 grid(T, (W + 255) / 256);
+  const bool vec = W % 4 == 0 && h_stride % 4 == 0 && shared_stride % 4 == 0 &&
+                   (((uintptr_t)out | (uintptr_t)ys | (uintptr_t)h | (uintptr_t)shared) & 15) == 0;
+  const dim3 grid(T, vec ? (W / 4 + 255) / 256 : (W + 255) / 256);
   if (grid.y > 65535) return -3;
-  if (is_f32)
-    moe_combine_kernel<float><<<grid, 256, 0, s>>>((float*)out, (const float*)ys, where, (const float*)h, h_stride, idx, wts,
-                                                   (const float*)shared, shared_stride, E, top, W);
-  else
-    moe_combine_kernel<uint16_t><<<grid, 256, 0, s>>>((uint16_t*)out, (const uint16_t*)ys, where, (const uint16_t*)h,
-                                                      h_stride, idx, wts, (const uint16_t*)shared, shared_stride, E, top, W);
+#define DGI_COMB(TT_, VV_)                                                                                          \
+  moe_combine_kernel<TT_, VV_><<<grid, 256, 0, s>>>((TT_*)out, (const TT_*)ys, where, (const TT_*)h, h_stride, idx, wts, \
+                                                    (const TT_*)shared, shared_stride, E, top, W)
+  if (is_f32) { if (vec) DGI_COMB(float, 4); else DGI_COMB(float, 1); }
+  else { if (vec) DGI_COMB(uint16_t, 4); else DGI_COMB(uint16_t, 1); }
+#undef DGI_COMB
   DGI_CHECK_LAUNCH();
   return 0;
 }

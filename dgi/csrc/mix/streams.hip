@@ -24,6 +24,17 @@ template <typename T> __device__ __forceinline__ float ldf(const T* p);
 template <> __device__ __forceinline__ float ldf<float>(const float* p) { return *p; }
 template <> __device__ __forceinline__ float ldf<uint16_t>(const uint16_t* p) { return bf16_to_f32(*p); }
 
+template <typename T> __device__ __forceinline__ void ld4(const T* p, float* f);
+template <> __device__ __forceinline__ void ld4<float>(const float* p, float* f) {
+  const float4 v = *reinterpret_cast<const float4*>(p);
+  f[0] = v.x; f[1] = v.y; f[2] = v.z; f[3] = v.w;
+}
+template <> __device__ __forceinline__ void ld4<uint16_t>(const uint16_t* p, float* f) {
+  const uint2 v = *reinterpret_cast<const uint2*>(p);
+  f[0] = __uint_as_float(v.x << 16); f[1] = __uint_as_float(v.x & 0xffff0000u);
+  f[2] = __uint_as_float(v.y << 16); f[3] = __uint_as_float(v.y & 0xffff0000u);
+}
+
 constexpr int MAXS = 8;      // streams
 
 __device__ __forceinline__ float block_sum(float v, float* red) {
@@ -77,7 +88,9 @@ __global__ void store_last_token_kernel(int* __restrict__ prev_tok, const int* _
   if (r1 > r0) prev_tok[seq_slots[i]] = ids[r1 - 1];
 }
 
-template <typename T>
+// V = 4: four consecutive columns per thread (16-byte stream accesses; W, strides and pointers allow it),
+// V = 1: any width.  The arithmetic per column is the same.
+template <typename T, int V>
 __global__ __launch_bounds__(256) void hc_mix_norm_kernel(
     float* __restrict__ xs, int S, int NT, int W, const T* __restrict__ y, int y_stride, const T* __restrict__ gate,
     int gate_stride, const float* __restrict__ gate_b, const float* __restrict__ mixm, const float* __restrict__ outc,
@@ -94,36 +107,66 @@ __global__ __launch_bounds__(256) void hc_mix_norm_kernel(
   }
   __syncthreads();
   float sum = 0.f;
-  for (int w = threadIdx.x; w < W; w += blockDim.x) {
-    float x[MAXS];
+  for (int w = threadIdx.x * V; w < W; w += blockDim.x * V) {
+    float x[MAXS][V];
 #pragma unroll
-    for (int s = 0; s < MAXS; ++s) x[s] = s < S ? xs[((size_t)s * NT + row) * W + w] : 0.f;
+    for (int s = 0; s < MAXS; ++s) {
+      if (s < S) {
+        if constexpr (V == 4) ld4<float>(xs + ((size_t)s * NT + row) * W + w, x[s]);
+        else x[s][0] = xs[((size_t)s * NT + row) * W + w];
+      } else {
+#pragma unroll
+        for (int k = 0; k < V; ++k) x[s][k] = 0.f;
+      }
+    }
     if (y) {
-      float yy = ldf<T>(y + (size_t)row * y_stride + w);
-      if (gate) yy *= 1.f / (1.f + expf(-(ldf<T>(gate + (size_t)row * gate_stride + w) + gate_b[w])));
-      float nx[MAXS];
+      float yy[V], gg[V], gb[V];
+      if constexpr (V == 4) {
+        ld4<T>(y + (size_t)row * y_stride + w, yy);
+        if (gate) { ld4<T>(gate + (size_t)row * gate_stride + w, gg); ld4<float>(gate_b + w, gb); }
+      } else {
+        yy[0] = ldf<T>(y + (size_t)row * y_stride + w);
+        if (gate) { gg[0] = ldf<T>(gate + (size_t)row * gate_stride + w); gb[0] = gate_b[w]; }
+      }
+      if (gate) {
+#pragma unroll
+        for (int k = 0; k < V; ++k) yy[k] *= 1.f / (1.f + expf(-(gg[k] + gb[k])));
+      }
+      float nx[MAXS][V];
 #pragma unroll
       for (int t = 0; t < MAXS; ++t) {
-        float a = 0.f;
-        if (t < S) {
 #pragma unroll
-          for (int s = 0; s < MAXS; ++s)
-            if (s < S) a += cm[s * S + t] * x[s];
-          a += co[t] * yy;
-          xs[((size_t)t * NT + row) * W + w] = a;
+        for (int k = 0; k < V; ++k) {
+          float a = 0.f;
+          if (t < S) {
+#pragma unroll
+            for (int s = 0; s < MAXS; ++s)
+              if (s < S) a += cm[s * S + t] * x[s][k];
+            a += co[t] * yy[k];
+          }
+          nx[t][k] = a;
         }
-        nx[t] = a;
+        if (t < S) {
+          if constexpr (V == 4)
+            *reinterpret_cast<float4*>(xs + ((size_t)t * NT + row) * W + w) = make_float4(nx[t][0], nx[t][1], nx[t][2], nx[t][3]);
+          else xs[((size_t)t * NT + row) * W + w] = nx[t][0];
+        }
       }
 #pragma unroll
-      for (int t = 0; t < MAXS; ++t) x[t] = nx[t];
+      for (int t = 0; t < MAXS; ++t)
+#pragma unroll
+        for (int k = 0; k < V; ++k) x[t][k] = nx[t][k];
     }
     if (in_next) {
-      float u = 0.f;
 #pragma unroll
-      for (int s = 0; s < MAXS; ++s)
-        if (s < S) u += ci[s] * x[s];
-      us[w] = u;
-      sum += u;
+      for (int k = 0; k < V; ++k) {
+        float u = 0.f;
+#pragma unroll
+        for (int s = 0; s < MAXS; ++s)
+          if (s < S) u += ci[s] * x[s][k];
+        us[w + k] = u;
+        sum += u;
+      }
     }
   }
   if (!in_next) return;
@@ -176,14 +219,25 @@ extern "C" int dgi_hc_mix_norm(float* xs, int S, int T, int W, const void* y, in
   if (S < 1 || S > MAXS) return -2;
   if (W > 16384) return -3;
   const size_t lds = in_next ? (size_t)W * 4 : 0;
+  const bool vec = W % 4 == 0 && y_stride % 4 == 0 && gate_stride % 4 == 0 &&
+                   (((uintptr_t)xs | (uintptr_t)y | (uintptr_t)gate | (uintptr_t)gate_b) & 15) == 0;
   if (is_f32) {
     if (hd) return -4;
-    hc_mix_norm_kernel<float><<<T, 256, lds, s>>>(xs, S, T, W, (const float*)y, y_stride, (const float*)gate,
-                                                  gate_stride, gate_b, mixm, outc, in_next, norm_w, eps, h32, nullptr);
+    if (vec)
+      hc_mix_norm_kernel<float, 4><<<T, 256, lds, s>>>(xs, S, T, W, (const float*)y, y_stride, (const float*)gate,
+                                                       gate_stride, gate_b, mixm, outc, in_next, norm_w, eps, h32, nullptr);
+    else
+      hc_mix_norm_kernel<float, 1><<<T, 256, lds, s>>>(xs, S, T, W, (const float*)y, y_stride, (const float*)gate,
+                                                       gate_stride, gate_b, mixm, outc, in_next, norm_w, eps, h32, nullptr);
   } else {
-    hc_mix_norm_kernel<uint16_t><<<T, 256, lds, s>>>(xs, S, T, W, (const uint16_t*)y, y_stride, (const uint16_t*)gate,
-                                                     gate_stride, gate_b, mixm, outc, in_next, norm_w, eps, h32,
-                                                     (uint16_t*)hd);
+    if (vec)
+      hc_mix_norm_kernel<uint16_t, 4><<<T, 256, lds, s>>>(xs, S, T, W, (const uint16_t*)y, y_stride, (const uint16_t*)gate,
+                                                          gate_stride, gate_b, mixm, outc, in_next, norm_w, eps, h32,
+                                                          (uint16_t*)hd);
+    else
+      hc_mix_norm_kernel<uint16_t, 1><<<T, 256, lds, s>>>(xs, S, T, W, (const uint16_t*)y, y_stride, (const uint16_t*)gate,
+                                                          gate_stride, gate_b, mixm, outc, in_next, norm_w, eps, h32,
+                                                          (uint16_t*)hd);
   }
   DGI_CHECK_LAUNCH();
   return 0;

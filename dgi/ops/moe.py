@@ -8,10 +8,11 @@ and ``down`` [E, W, ff].
 
 Two evaluation paths on the GPU, same result up to summation order:
 
-* few rows (decode steps, and every step inside a captured graph): workgroups own (expert, output
-  tile) and walk the pairs that chose the expert, so each expert's rows stream from the stacked
-  weights once per handful of tokens (weight-bandwidth bound, no host round trip), then the combine
-  kernel;
+* few rows (decode steps, and every step inside a captured graph; no host round trip): when the step's
+  (token, route) pairs are at least as many as the experts, all experts run as one batched vendor GEMM
+  over the step's rows and the combine kernel picks each token's routes; with fewer pairs, workgroups own
+  (expert, output tile) and walk the pairs that chose the expert, so only the chosen experts' rows stream
+  from the stacked weights;
 * many rows (prompt portions): pairs are sorted by expert, every expert with tokens runs the
   vendor GEMM over its contiguous segment, and a combine kernel gathers each token's routes in
   their fixed order (deterministic, no atomics).
@@ -89,6 +90,16 @@ def moe_experts(h, idx, wts, gate_up, down, shared=None) -> torch.Tensor:
     top = idx.shape[1]
     out = torch.empty(T, W, dtype=h.dtype, device=h.device)
     if T <= EXPERT_MAJOR_ROWS or torch.cuda.is_current_stream_capturing():
+        if T * top >= E:
+            # a small step that touches (nearly) every expert anyway: all experts as one batched vendor GEMM
+            # over the step's rows (weight-bandwidth bound either way; the extra FLOPs are free at these
+            # sizes), then every token picks its routes' rows in the combine
+            gu = torch.matmul(h.unsqueeze(0), gate_up.transpose(1, 2))                  # [E, T, 2 ff]
+            act = silu_mul(gu.view(E * T, 2 * ff))
+            ys = torch.bmm(act.view(E, T, ff), down.transpose(1, 2)).view(E * T, W)
+            where = (idx * T + torch.arange(T, dtype=torch.int32, device=h.device)[:, None]).clamp_(0, E * T - 1)
+            _call("moe_combine", out, ys, where, h, idx, wts, shared, E)
+            return out
         mid = torch.empty(T * top, ff, dtype=torch.float32, device=h.device)
         ys = torch.empty(T * top, W, dtype=h.dtype, device=h.device)     # identity pairs' rows are never read
         _call("moe_expert_gate_up", mid, h, idx, gate_up)

@@ -223,20 +223,21 @@ def test_hyper_connection_update_and_norm(device, dtype, S, W):
 
 @pytest.mark.parametrize("device", DEVICES)
 @pytest.mark.parametrize("taps,act,residual", [(4, 0, True), (3, 1, False), (1, 0, True), (2, 1, True), (6, 0, False)])
-def test_causal_conv_portions(device, taps, act, residual):
+@pytest.mark.parametrize("C,pad,off", [(37, 6, 3), (40, 8, 4)])        # odd channels / the four-channel vector path
+def test_causal_conv_portions(device, taps, act, residual, C, pad, off):
     """A sequence cut into portions of 1, 2, taps - 1, taps and more rows, another one beside it,
     slots that held other data before: equal to the whole-sequence convolution."""
     g = torch.Generator().manual_seed(3)
-    C, n = 37, 23
+    n = 23
     w = torch.randn(C, taps, generator=g)
     b = torch.randn(C, generator=g) if act else None
-    xa, xb = torch.randn(n, C + 6, generator=g), torch.randn(n, C + 6, generator=g)       # wider rows: a column slice
+    xa, xb = torch.randn(n, C + pad, generator=g), torch.randn(n, C + pad, generator=g)   # wider rows: a column slice
     tail = torch.randn(5, max(taps - 1, 0), C).to(device) * 100 if taps > 1 else None     # stale slot contents
     want = {}
     for name, x in (("a", xa), ("b", xb)):
-        o = orc.causal_taps(x[:, 3:3 + C].double(), w.double(), None if b is None else b.double())
+        o = orc.causal_taps(x[:, off:off + C].double(), w.double(), None if b is None else b.double())
         o = orc.silu(o) if act else o
-        want[name] = o + x[:, 3:3 + C].double() if residual else o
+        want[name] = o + x[:, off:off + C].double() if residual else o
     cuts = [1, 1, 2, max(taps - 1, 1), taps, 5, 1, n]
     at_a = at_b = 0
     got_a, got_b = [], []
@@ -250,7 +251,7 @@ def test_causal_conv_portions(device, taps, act, residual):
         if not lens:
             break
         pos, rs, r0, sl = seq_meta(lens, starts, slots, device)
-        x = torch.cat(rows, 0).to(device)[:, 3:3 + C]
+        x = torch.cat(rows, 0).to(device)[:, off:off + C]
         out = recur.causal_conv(x, w.to(device), None if b is None else b.to(device), tail, pos, rs, r0, sl, act=act,
                                 residual=residual, out_dtype=torch.float32)
         if nb_:
@@ -387,8 +388,9 @@ def test_gated_group_norm_and_silu_mul(device, dtype):
         got = recur.gated_group_norm(y.to(device), zw.to(device)[:, 2:2 + C], w.to(device), groups, 1e-4, dtype)
         gv = (y.double() * orc.silu(z.double())).view(T, groups, C // groups)
         close(got, orc.unit_rms(gv, 1e-4).reshape(T, C) * w.double(), tol)
-    gu = torch.randn(T, 50, generator=g).to(dtype)
-    close(moe.silu_mul(gu.to(device)), orc.silu(gu[:, :25].double()) * gu[:, 25:].double(), tol)
+    for I in (25, 32):                                 # scalar path and the four-column vector path
+        gu = torch.randn(T, 2 * I, generator=g).to(dtype)
+        close(moe.silu_mul(gu.to(device)), orc.silu(gu[:, :I].double()) * gu[:, I:].double(), tol)
 
 
 @pytest.mark.parametrize("device", DEVICES)
@@ -470,7 +472,7 @@ def test_mfma_prompt_attention_with_distance_bias(hd, H, G):
 
 @pytest.mark.parametrize("device", DEVICES)
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("T,E,I,top", [(5, 6, 3, 3), (70, 6, 3, 3), (9, 4, 0, 1), (40, 2, 2, 4), (3, 70, 0, 8), (300, 3, 1, 2)])
+@pytest.mark.parametrize("T,E,I,top", [(5, 6, 3, 3), (70, 6, 3, 3), (9, 4, 0, 1), (40, 2, 2, 4), (3, 70, 0, 8), (2, 16, 2, 3), (300, 3, 1, 2)])
 def test_moe_routing_and_experts(device, dtype, T, E, I, top):
     g = torch.Generator().manual_seed(7)
     W, ff = 48, 20
