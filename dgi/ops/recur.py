@@ -3,7 +3,7 @@ hashed-bigram + position embedding, hyper-connected stream mixing fused with the
 causal convolutions over packed rows with their tails in state slots, the Mamba-2 selective scan
 and its gated group norm.
 
-Same contract as ``dgi.ops.mix``: GPU tensors run the HIP kernel (and raise if the library is
+Same rules as ``dgi.ops.mix``: GPU tensors run the HIP kernel (and raise if the library is
 missing), CPU tensors the ``*_ref`` function in fp32, which is also the kernel tests' oracle.
 
 Rows of a step are ``[decode rows | prompt portions]``; ``row_seq`` [T] names each row's sequence
