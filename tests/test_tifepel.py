@@ -49,11 +49,11 @@ def small_cfg(**kw) -> TifepelConfig:
     return TifepelConfig(**args)
 
 
-def engine(cfg, device, dtype=torch.float32, num_blocks=96, bs=4, seed=3, max_len=256, seqs=4):
+def engine(cfg, device, dtype=torch.float32, num_blocks=96, bs=4, seed=3, max_len=256, seqs=4, graphs=False):
     return LLMEngine(EngineConfig(model="tifepel-test", device=device, dtype=dtype, block_size=bs, num_blocks=num_blocks,
                                   max_num_seqs=seqs, max_model_len=max_len, max_num_batched_tokens=max_len,
-                                  enable_prefix_caching=True, use_graphs=False, token_align=0, decode_lookahead=False,
-                                  seed=seed), model_cfg=copy.deepcopy(cfg))
+                                  enable_prefix_caching=True, use_graphs=graphs, token_align=0, decode_lookahead=graphs,
+                                  seed=seed, graph_buckets=(1, 2, 4) if graphs else None), model_cfg=copy.deepcopy(cfg))
 
 
 def toks(n, seed=0, vocab=53):
@@ -611,6 +611,48 @@ def test_greedy_generation_through_the_scheduler(device):
             assert tok == int(lg.argmax()) or (top2[0] - top2[1]) < 1e-3
             seq.append(tok)
     assert eng.pool.num_used == 0 and eng.state_pool.num_free == 4
+
+
+@pytest.mark.gpu
+def test_graph_decode_equals_eager_decode():
+    """Decode steps replayed as hipGraphs (state slots in the staging image, padded rows on the reserved
+    slot, decode lookahead) produce the tokens of the eager engine; replays follow each other with
+    eager prompt steps between them."""
+    cfg = small_cfg()
+    eager, graph = engine(cfg, "cuda", max_len=128), engine(cfg, "cuda", max_len=128, graphs=True)
+    graph.model.copy_from(eager.model)
+    prompts = [toks(9, 60), toks(17, 61), toks(3, 62)]
+    sp = SamplingParams(max_tokens=14, temperature=0.0, ignore_eos=True)
+    want = [r.output for r in eager.generate(prompts, sp)]
+    for _ in range(2):                                       # a second batch reuses slots and replays again
+        assert [r.output for r in graph.generate(prompts, sp)] == want
+    assert graph.runner.graphs is not None and graph.runner.graphs.captured
+    assert graph.state_pool.num_free == 4 and graph.pool.num_used == 0
+
+
+@pytest.mark.gpu
+def test_mfma_prompt_path_in_the_model(monkeypatch):
+    """Layers whose bf16 heads are 64 / 128 wide take the MFMA prompt kernel: same logits as the
+    row-wise kernel on the same engine (portions on top of cached tokens, two prompts in one step);
+    no experts, so nothing can flip a routing decision."""
+    cfg = TifepelConfig(name="t", vocab_size=53, hidden_size=64, layers=[
+        LayerSpec("attention", attn(4, 2, 64, 64, 0.125, 0.3, 16, 10, 40.0), None),
+        LayerSpec("mamba2", Mamba2Spec(2, 16, 16, 1, 4, 1), None),
+        LayerSpec("attention", attn(2, 1, 128, 128, 0.09, 0.0, 0, 8, 200.0), None),
+    ], streams=2, canon_taps=4, bigram_buckets=29, bigram_mul_prev=5, bigram_mul_cur=3, max_position=512)
+    a, b = toks(200, 70), toks(90, 71)
+
+    def run():
+        eng = engine(cfg, "cuda", dtype=torch.bfloat16, num_blocks=64, bs=16, max_len=512)
+        out = [eng.feed([("a", a[:150], list(range(150)))]),
+               eng.feed([("a", a[150:], list(range(50))), ("b", b, list(range(90)))], ["a", "b"])]
+        return torch.cat([o for step in out for o in step], 0)
+
+    assert mix.masked_prefill_available()
+    fast = run()
+    monkeypatch.setattr(mix, "MASKED_PREFILL", False)
+    slow = run()
+    close(fast, slow, 0.06 * max(1.0, slow.abs().max().item()))
 
 
 def test_preempted_sequence_recomputes_its_state():
