@@ -12,8 +12,8 @@
 // not depend on how a prompt was cut.  x | B | C come as one fp32 row (the convolution's output).
 //
 // Work split: a workgroup owns (sequence, head, 16 value columns); thread (column v, n-lane l) keeps
-// S[n][v] for n = 4 l + 64 q + j in registers, so the y reduction over n is four shuffles inside a
-// 16-lane group.  The serial loop over tokens never waits for global memory: B, C, x and the step
+// S[n][v] for n = 4 l + 64 q + j in registers, so the y reduction over n is four DPP rotate-adds inside a
+// 16-lane row.  The serial loop over tokens never waits for global memory: B, C, x and the step
 // sizes of 16 tokens are staged in LDS (the next tile's loads are in flight, in registers, while the
 // current one is consumed; softplus and the decay are computed once per token while staging), and a
 // token costs two 16-byte LDS reads per four state values.  The state is stored value-major,
@@ -34,6 +34,17 @@ template <> __device__ __forceinline__ float ldf<uint16_t>(const uint16_t* p) { 
 template <typename T> __device__ __forceinline__ void stf(T* p, float v);
 template <> __device__ __forceinline__ void stf<float>(float* p, float v) { *p = v; }
 template <> __device__ __forceinline__ void stf<uint16_t>(uint16_t* p, float v) { *p = f32_to_bf16(v); }
+
+// Sum over the 16 lanes of a DPP row (lanes 16 r .. 16 r + 15), result in every lane: four rotate-and-add
+// steps in the VALU (row_ror 8, 4, 2, 1) — no trip through the LDS permute unit, which a per-token
+// reduction inside a serial loop would otherwise wait for four times.
+__device__ __forceinline__ float row16_sum(float v) {
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x128, 0xf, 0xf, false));
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x124, 0xf, 0xf, false));
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x122, 0xf, 0xf, false));
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x121, 0xf, 0xf, false));
+  return v;
+}
 
 constexpr int COLS = 16;     // value columns per workgroup
 constexpr int NL = 16;       // n-lanes per column
@@ -138,8 +149,7 @@ __global__ __launch_bounds__(COLS * NL) void ssm_scan_kernel(
         acc += S[q][0] * c4.x + S[q][1] * c4.y + S[q][2] * c4.z + S[q][3] * c4.w;
       }
       if (mode != 1) {                                   // mode 1: chunk states only, no outputs
-#pragma unroll
-        for (int o = NL / 2; o > 0; o >>= 1) acc += __shfl_xor(acc, o, 64);
+        acc = row16_sum(acc);
         if (l == 0 && vok) y[(size_t)(t0 + k) * inner + (size_t)h * dv + v] = acc + dsk * xv;
       }
     }
