@@ -55,7 +55,7 @@ __global__ __launch_bounds__(256) void causal_conv_kernel(
 }
 
 // Four channels per thread: 16-byte (fp32) / 8-byte (bf16) row accesses and the thread's 4 x taps
-// weights as contiguous 16-byte loads.  Same arithmetic, per channel, in the same order.
+// weights as contiguous 16-byte loads.  Same arithmetic per channel.
 template <typename T> __device__ __forceinline__ void ld4(const T* p, float* f);
 template <> __device__ __forceinline__ void ld4<float>(const float* p, float* f) {
   const float4 v = *reinterpret_cast<const float4*>(p);
@@ -74,45 +74,57 @@ template <> __device__ __forceinline__ void st4<uint16_t>(uint16_t* p, const flo
   *reinterpret_cast<uint2*>(p) = make_uint2(pack_bf16x2(f[0], f[1]), pack_bf16x2(f[2], f[3]));
 }
 
+// A thread walks `rpw` consecutive rows with the last TAPS - 1 inputs of its channels in registers: inside a
+// sequence's portion every input is read once (rows of a portion are consecutive positions); at the first row of
+// the walk and wherever a new sequence starts the window is loaded afresh (rows of the step or the slot's tail).
 template <typename TI, typename TO, int TAPS>
 __global__ __launch_bounds__(256) void causal_conv_vec_kernel(
-    TO* __restrict__ out, const TI* __restrict__ x, int x_stride, int C, const float* __restrict__ w,
+    TO* __restrict__ out, const TI* __restrict__ x, int x_stride, int T, int C, const float* __restrict__ w,
     const float* __restrict__ bias, const float* __restrict__ tail, const int* __restrict__ positions,
     const int* __restrict__ row_seq, const int* __restrict__ seq_row0, const int* __restrict__ seq_slots, int act,
-    int residual) {
-  const int row = blockIdx.x;
+    int residual, int rpw) {
   const int c = (blockIdx.y * blockDim.x + threadIdx.x) * 4;
   if (c >= C) return;
-  const int seq = row_seq[row];
-  const int r0 = seq_row0[seq];
-  const int pos = positions[row], p0 = positions[r0];
-  const float* tl = tail ? tail + (size_t)seq_slots[seq] * (TAPS - 1) * C : nullptr;
   float wv[4 * TAPS];
 #pragma unroll
   for (int i = 0; i < TAPS; ++i) ld4<float>(w + (size_t)c * TAPS + 4 * i, wv + 4 * i);     // wv[ch * TAPS + j]
-  float acc[4] = {0.f, 0.f, 0.f, 0.f};
-  if (bias) ld4<float>(bias + c, acc);
-  float cur[4] = {0.f, 0.f, 0.f, 0.f};
+  float bv[4] = {0.f, 0.f, 0.f, 0.f};
+  if (bias) ld4<float>(bias + c, bv);
+  float win[TAPS][4];                                  // win[j]: input at position pos - (TAPS - 1) + j
+  const int row_begin = blockIdx.x * rpw, row_end = min(T, row_begin + rpw);
+  for (int row = row_begin; row < row_end; ++row) {
+    const int seq = row_seq[row];
+    const int r0 = seq_row0[seq];
+    if (row == row_begin || row == r0) {               // load the older inputs
+      const int pos = positions[row], p0 = positions[r0];
+      const float* tl = tail ? tail + (size_t)seq_slots[seq] * (TAPS - 1) * C : nullptr;
 #pragma unroll
-  for (int j = 0; j < TAPS; ++j) {
-    const int pp = pos - (TAPS - 1) + j;
-    if (pp < 0) continue;
-    float v[4];
-    if (pp >= p0) ld4<TI>(x + (size_t)(r0 + pp - p0) * x_stride + c, v);
-    else ld4<float>(tl + (size_t)(pp - (p0 - (TAPS - 1))) * C + c, v);
+      for (int j = 0; j < TAPS - 1; ++j) {
+        const int pp = pos - (TAPS - 1) + j;
 #pragma unroll
-    for (int ch = 0; ch < 4; ++ch) acc[ch] += wv[ch * TAPS + j] * v[ch];
-    if (j == TAPS - 1) {
+        for (int ch = 0; ch < 4; ++ch) win[j][ch] = 0.f;
+        if (pp >= p0) ld4<TI>(x + (size_t)(r0 + pp - p0) * x_stride + c, win[j]);
+        else if (pp >= 0) ld4<float>(tl + (size_t)(pp - (p0 - (TAPS - 1))) * C + c, win[j]);
+      }
+    } else {
 #pragma unroll
-      for (int ch = 0; ch < 4; ++ch) cur[ch] = v[ch];
+      for (int j = 0; j < TAPS - 1; ++j)
+#pragma unroll
+        for (int ch = 0; ch < 4; ++ch) win[j][ch] = win[j + 1][ch];
     }
-  }
+    ld4<TI>(x + (size_t)row * x_stride + c, win[TAPS - 1]);
+    float acc[4];
 #pragma unroll
-  for (int ch = 0; ch < 4; ++ch) {
-    if (act == 1) acc[ch] = acc[ch] / (1.f + expf(-acc[ch]));
-    if (residual) acc[ch] += cur[ch];
+    for (int ch = 0; ch < 4; ++ch) {
+      float a = bv[ch];
+#pragma unroll
+      for (int j = 0; j < TAPS; ++j) a += wv[ch * TAPS + j] * win[j][ch];
+      if (act == 1) a = a / (1.f + expf(-a));
+      if (residual) a += win[TAPS - 1][ch];
+      acc[ch] = a;
+    }
+    st4<TO>(out + (size_t)row * C + c, acc);
   }
-  st4<TO>(out + (size_t)row * C + c, acc);
 }
 
 template <typename TI>
@@ -156,10 +168,11 @@ extern "C" int dgi_causal_conv(void* out, int out_f32, const void* x, int x_f32,
   const bool vec = C % 4 == 0 && x_stride % 4 == 0 && taps >= 2 && taps <= 4 &&
                    (((uintptr_t)x | (uintptr_t)out | (uintptr_t)w | (uintptr_t)bias | (uintptr_t)tail) & 15) == 0;
   if (vec) {
-    const dim3 vgrid(T, (C / 4 + 255) / 256);
+    const int rpw = T >= 2048 ? 8 : 1;                 // rows per thread walk: large steps only (small ones need the workgroups)
+    const dim3 vgrid((T + rpw - 1) / rpw, (C / 4 + 255) / 256);
 #define DGI_CONVV(TI, TO, TP)                                                                                      \
-  causal_conv_vec_kernel<TI, TO, TP><<<vgrid, 256, 0, s>>>((TO*)out, (const TI*)x, x_stride, C, w, bias, tail,     \
-                                                          positions, row_seq, seq_row0, seq_slots, act, residual)
+  causal_conv_vec_kernel<TI, TO, TP><<<vgrid, 256, 0, s>>>((TO*)out, (const TI*)x, x_stride, T, C, w, bias, tail,  \
+                                                          positions, row_seq, seq_row0, seq_slots, act, residual, rpw)
 #define DGI_CONVT(TI, TO) \
   do { if (taps == 2) DGI_CONVV(TI, TO, 2); else if (taps == 3) DGI_CONVV(TI, TO, 3); else DGI_CONVV(TI, TO, 4); } while (0)
     if (x_f32 && out_f32) DGI_CONVT(float, float);

@@ -263,6 +263,29 @@ def test_causal_conv_portions(device, taps, act, residual, C, pad, off):
     close(torch.cat(got_b, 0), want["b"][:at_b], 1e-4)
 
 
+@pytest.mark.gpu
+@pytest.mark.parametrize("taps,dtype", [(4, torch.float32), (3, torch.bfloat16), (2, torch.float32)])
+def test_causal_conv_large_step_walks_rows(taps, dtype):
+    """Steps of 2048 rows and more let a thread walk several consecutive rows with the window in registers:
+    sequences that start inside a walk, one-row sequences, continued portions with their tails, a fresh one."""
+    g = torch.Generator().manual_seed(11)
+    C = 40
+    lens, starts, slots = [1000, 1, 700, 3, 397, 5], [0, 9, 50, 0, 2, 1], [1, 2, 3, 4, 5, 6]
+    T = sum(lens)
+    assert T >= 2048
+    x = torch.randn(T, C + 8, generator=g).to(dtype)
+    w, b = torch.randn(C, taps, generator=g), torch.randn(C, generator=g)
+    tail = torch.randn(8, taps - 1, C, generator=g)
+    pos, rs, r0, sl = seq_meta(lens, starts, slots, "cpu")
+    t_ref = tail.clone()
+    want = recur.causal_conv_ref(x[:, 4:4 + C], w, b, t_ref, pos, r0, sl, 1, True, torch.float32)
+    t_gpu = tail.clone().cuda()
+    got = recur.causal_conv(x.cuda()[:, 4:4 + C], w.cuda(), b.cuda(), t_gpu, pos.cuda(), rs.cuda(), r0.cuda(), sl.cuda(),
+                            act=1, residual=True, out_dtype=torch.float32)
+    close(got, want, 1e-4)
+    close(t_gpu[slots], t_ref[slots], 1e-6)
+
+
 def mamba_parts(g, heads, dv, N, G, T, dtype):
     inner = heads * dv
     xbc = torch.randn(T, inner + 2 * G * N, generator=g)
