@@ -219,6 +219,68 @@ __global__ __launch_bounds__(256) void gated_group_norm_kernel(
   }
 }
 
+template <typename T> __device__ __forceinline__ void ld4(const T* p, float* f);
+template <> __device__ __forceinline__ void ld4<float>(const float* p, float* f) {
+  const float4 v = *reinterpret_cast<const float4*>(p);
+  f[0] = v.x; f[1] = v.y; f[2] = v.z; f[3] = v.w;
+}
+template <> __device__ __forceinline__ void ld4<uint16_t>(const uint16_t* p, float* f) {
+  const uint2 v = *reinterpret_cast<const uint2*>(p);
+  f[0] = __uint_as_float(v.x << 16); f[1] = __uint_as_float(v.x & 0xffff0000u);
+  f[2] = __uint_as_float(v.y << 16); f[3] = __uint_as_float(v.y & 0xffff0000u);
+}
+template <typename T> __device__ __forceinline__ void st4(T* p, const float* f);
+template <> __device__ __forceinline__ void st4<float>(float* p, const float* f) {
+  *reinterpret_cast<float4*>(p) = make_float4(f[0], f[1], f[2], f[3]);
+}
+template <> __device__ __forceinline__ void st4<uint16_t>(uint16_t* p, const float* f) {
+  *reinterpret_cast<uint2*>(p) = make_uint2(pack_bf16x2(f[0], f[1]), pack_bf16x2(f[2], f[3]));
+}
+
+// One pass: a group of up to 256 * 4 * VPT values stays in registers between the sum of squares and the
+// store (y and z are read once); groups in fours of columns, 16-byte accesses.
+template <typename TZ, typename TO, int VPT>
+__global__ __launch_bounds__(256) void gated_group_norm_reg_kernel(
+    TO* __restrict__ out, const float* __restrict__ y, const TZ* __restrict__ z, int z_stride,
+    const float* __restrict__ w, int C, int groups, float eps) {
+  __shared__ float red[4];
+  const int row = blockIdx.x, grp = blockIdx.y;
+  const int gs = C / groups;
+  const float* yp = y + (size_t)row * C + (size_t)grp * gs;
+  const TZ* zp = z + (size_t)row * z_stride + (size_t)grp * gs;
+  float gv[VPT][4];
+  float ss = 0.f;
+#pragma unroll
+  for (int i = 0; i < VPT; ++i) {
+    const int c = (threadIdx.x + 256 * i) * 4;
+    if (c < gs) {
+      float yy[4], zz[4];
+      ld4<float>(yp + c, yy);
+      ld4<TZ>(zp + c, zz);
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        gv[i][k] = yy[k] * zz[k] / (1.f + expf(-zz[k]));
+        ss += gv[i][k] * gv[i][k];
+      }
+    }
+  }
+  ss = wave_sum(ss);
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = ss;
+  __syncthreads();
+  const float r = 1.f / sqrtf((red[0] + red[1] + red[2] + red[3]) / (float)gs + eps);
+#pragma unroll
+  for (int i = 0; i < VPT; ++i) {
+    const int c = (threadIdx.x + 256 * i) * 4;
+    if (c < gs) {
+      float ww[4], o[4];
+      ld4<float>(w + (size_t)grp * gs + c, ww);
+#pragma unroll
+      for (int k = 0; k < 4; ++k) o[k] = gv[i][k] * r * ww[k];
+      st4<TO>(out + (size_t)row * C + (size_t)grp * gs + c, o);
+    }
+  }
+}
+
 }  // namespace
 
 // ws / wsd: workspace for the chunked form ([n_seq * nchunks][heads][dv][N] states and [n_seq * nchunks][heads]
@@ -270,6 +332,23 @@ extern "C" int dgi_gated_group_norm(void* out, int out_f32, const float* y, cons
   if (T == 0) return 0;
   if (groups <= 0 || C % groups || groups > 65535) return -2;
   const dim3 grid(T, groups);
+  const int gs = C / groups;
+  if (gs % 4 == 0 && gs <= 256 * 4 * 8 && z_stride % 4 == 0 &&
+      (((uintptr_t)out | (uintptr_t)y | (uintptr_t)z | (uintptr_t)w) & 15) == 0 && z_f32 == out_f32) {
+    if (z_f32) {
+      if (gs <= 256 * 4 * 2)
+        gated_group_norm_reg_kernel<float, float, 2><<<grid, 256, 0, s>>>((float*)out, y, (const float*)z, z_stride, w, C, groups, eps);
+      else
+        gated_group_norm_reg_kernel<float, float, 8><<<grid, 256, 0, s>>>((float*)out, y, (const float*)z, z_stride, w, C, groups, eps);
+    } else {
+      if (gs <= 256 * 4 * 2)
+        gated_group_norm_reg_kernel<uint16_t, uint16_t, 2><<<grid, 256, 0, s>>>((uint16_t*)out, y, (const uint16_t*)z, z_stride, w, C, groups, eps);
+      else
+        gated_group_norm_reg_kernel<uint16_t, uint16_t, 8><<<grid, 256, 0, s>>>((uint16_t*)out, y, (const uint16_t*)z, z_stride, w, C, groups, eps);
+    }
+    DGI_CHECK_LAUNCH();
+    return 0;
+  }
   if (z_f32 && out_f32)
     gated_group_norm_kernel<float, float><<<grid, 256, 0, s>>>((float*)out, y, (const float*)z, z_stride, w, C, groups, eps);
   else if (!z_f32 && !out_f32)

@@ -404,13 +404,17 @@ def test_scan_remembers_a_far_token(device, dtype):
 def test_gated_group_norm_and_silu_mul(device, dtype):
     g = torch.Generator().manual_seed(5)
     T, C = 7, 96
-    y, zw, w = torch.randn(T, C, generator=g) * 3, torch.randn(T, C + 5, generator=g).to(dtype), torch.randn(C, generator=g)
-    z = zw[:, 2:2 + C]
     tol = 2e-5 if dtype == torch.float32 else 4e-2
-    for groups in (1, 3, 96):
-        got = recur.gated_group_norm(y.to(device), zw.to(device)[:, 2:2 + C], w.to(device), groups, 1e-4, dtype)
-        gv = (y.double() * orc.silu(z.double())).view(T, groups, C // groups)
-        close(got, orc.unit_rms(gv, 1e-4).reshape(T, C) * w.double(), tol)
+    for pad, off in ((5, 2), (16, 8)):                 # an unaligned column slice, and the aligned one-pass path
+        y, zw, w = torch.randn(T, C, generator=g) * 3, torch.randn(T, C + pad, generator=g).to(dtype), torch.randn(C, generator=g)
+        z = zw[:, off:off + C]
+        for groups in (1, 3, 96):
+            got = recur.gated_group_norm(y.to(device), zw.to(device)[:, off:off + C], w.to(device), groups, 1e-4, dtype)
+            gv = (y.double() * orc.silu(z.double())).view(T, groups, C // groups)
+            close(got, orc.unit_rms(gv, 1e-4).reshape(T, C) * w.double(), tol)
+    y, zw, w = torch.randn(3, 4096, generator=g), torch.randn(3, 4096, generator=g).to(dtype), torch.randn(4096, generator=g)
+    got = recur.gated_group_norm(y.to(device), zw.to(device), w.to(device), 1, 1e-4, dtype)       # eight chunks a thread
+    close(got, orc.unit_rms((y.double() * orc.silu(zw.double())).view(3, 1, 4096), 1e-4).reshape(3, 4096) * w.double(), tol)
     for I in (25, 32):                                 # scalar path and the four-column vector path
         gu = torch.randn(T, 2 * I, generator=g).to(dtype)
         close(moe.silu_mul(gu.to(device)), orc.silu(gu[:, :I].double()) * gu[:, I:].double(), tol)
@@ -555,12 +559,15 @@ def test_layer_streams_match_oracle(device):
 
 
 @pytest.mark.parametrize("device", DEVICES)
-@pytest.mark.parametrize("variant", ["base", "one_stream", "no_loop", "wide_taps", "loop3"])
+@pytest.mark.parametrize("variant", ["base", "one_stream", "no_loop", "wide_taps", "loop3", "all_mamba", "all_attention"])
 def test_whole_decode_and_portions_match_oracle(device, variant):
     """Whole prompt, token by token, and portions of several sizes (down to two tokens, across pages):
     all equal the oracle; other stream counts, tap counts and loop settings too."""
     kw = {"base": {}, "one_stream": {"streams": 1, "canon_taps": 1}, "no_loop": {"loop_times": 1},
-          "wide_taps": {"canon_taps": 5, "streams": 3}, "loop3": {"loop_start": 0, "loop_stop": 1, "loop_times": 3}}[variant]
+          "wide_taps": {"canon_taps": 5, "streams": 3}, "loop3": {"loop_start": 0, "loop_stop": 1, "loop_times": 3},
+          "all_mamba": {"layers": [l for l in small_cfg().layers if l.type == "mamba2"], "loop_start": 0, "loop_stop": 2},
+          "all_attention": {"layers": [l for l in small_cfg().layers if l.type == "attention"], "loop_start": 1,
+                            "loop_stop": 2}}[variant]
     eng = engine(small_cfg(**kw), device)
     t = toks(45, 2)
     want = oracle_logits(eng, t)
