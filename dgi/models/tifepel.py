@@ -331,8 +331,7 @@ class TifepelModel:
         pend = None                # (y, gate, gate bias, mix, out) of the sublayer whose update is due
         for r, li in enumerate(self.runs):
             L = self.layers[li]
-            subs = (("1", None), ("2", None)) if L.spec.mlp is not None else (("1", None),)
-            for q, _ in subs:
+            for q in ("1", "2") if L.spec.mlp is not None else ("1",):
                 h32, hd = recur.hc_mix_norm(xs, *(pend or (None, None, None, None, None)),
                                             getattr(L, f"hc{q}_in"), getattr(L, "norm" + q), eps, dt)
                 gate = ops.linear(hd, getattr(L, "rg" + q))
